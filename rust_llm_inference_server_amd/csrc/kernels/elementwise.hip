@@ -23,23 +23,23 @@ RLIS_API const char* rlis_last_error() { return g_err; }
 // ------------------------------------------------------------------------ embedding
 template <typename TW>
 __global__ void embed_kernel(float* __restrict__ out, const TW* __restrict__ table,
-                             const int* __restrict__ ids, int H) {
+                             const int* __restrict__ ids, int H, float scale) {
   const int t = blockIdx.x;
   const long long row = ids[t];
   const TW* src = table + row * H;
   float* dst = out + (long long)t * H;
-  for (int j = threadIdx.x; j < H; j += blockDim.x) dst[j] = ld(src + j);
+  for (int j = threadIdx.x; j < H; j += blockDim.x) dst[j] = ld(src + j) * scale;
 }
 
-// out (T,H) f32 <- table[ids] ; ids are checked against V on the host before the call.
+// out (T,H) f32 <- table[ids] * scale ; ids are checked against V on the host before the call.
 RLIS_API int rlis_embed(float* out, const void* table, int table_dtype, const int* ids, int T,
-                        int H, hipStream_t stream) {
+                        int H, float scale, hipStream_t stream) {
   RLIS_REQUIRE(T >= 0 && H > 0, "embed: bad sizes T=%d H=%d", T, H);
   if (T == 0) return 0;
   if (table_dtype == RLIS_F32)
-    embed_kernel<float><<<T, 256, 0, stream>>>(out, (const float*)table, ids, H);
+    embed_kernel<float><<<T, 256, 0, stream>>>(out, (const float*)table, ids, H, scale);
   else if (table_dtype == RLIS_BF16)
-    embed_kernel<bf16_t><<<T, 256, 0, stream>>>(out, (const bf16_t*)table, ids, H);
+    embed_kernel<bf16_t><<<T, 256, 0, stream>>>(out, (const bf16_t*)table, ids, H, scale);
   else
     RLIS_REQUIRE(false, "embed: unknown table dtype %d", table_dtype);
   RLIS_LAUNCH_CHECK("embed");
@@ -51,25 +51,28 @@ RLIS_API int rlis_embed(float* out, const void* table, int table_dtype, const in
 // added in order (and their sum rounded to bfloat16 first when round_parts is set).
 template <typename TD>
 __global__ void add_residual_kernel(float* __restrict__ resid, const TD* __restrict__ delta,
-                                    long long n, int parts, int round_parts) {
+                                    long long n, int parts, int round_parts,
+                                    float delta_scale) {
   long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   const long long stride = (long long)gridDim.x * blockDim.x;
   for (; i < n; i += stride) {
-    resid[i] += delta_sum(delta + i, parts, n, round_parts);
+    resid[i] += delta_scale * delta_sum(delta + i, parts, n, round_parts);
   }
 }
 
+// resid += delta_scale * delta (the multiplier of a block's output, in float32).
 RLIS_API int rlis_add_residual(float* resid, const void* delta, int delta_dtype, long long n,
-                               int parts, int round_parts, hipStream_t stream) {
+                               int parts, int round_parts, float delta_scale,
+                               hipStream_t stream) {
   RLIS_REQUIRE(parts >= 1, "add_residual: parts=%d", parts);
   if (n <= 0) return 0;
   const int blocks = (int)(ceil_div_ll(n, 256) < 4096 ? ceil_div_ll(n, 256) : 4096);
   if (delta_dtype == RLIS_F32)
     add_residual_kernel<float><<<blocks, 256, 0, stream>>>(resid, (const float*)delta, n, parts,
-                                                           round_parts);
+                                                           round_parts, delta_scale);
   else if (delta_dtype == RLIS_BF16)
     add_residual_kernel<bf16_t><<<blocks, 256, 0, stream>>>(resid, (const bf16_t*)delta, n, parts,
-                                                            round_parts);
+                                                            round_parts, delta_scale);
   else
     RLIS_REQUIRE(false, "add_residual: unknown dtype %d", delta_dtype);
   RLIS_LAUNCH_CHECK("add_residual");
@@ -87,7 +90,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restri
                                    const TW* __restrict__ weight, TO* __restrict__ out,
                                    const int* __restrict__ rows, int H, float eps,
                                    int write_resid, int parts, long long part_stride,
-                                   int round_parts) {
+                                   int round_parts, float delta_scale) {
   __shared__ float red[NT / kWave];
   const int r = blockIdx.x;
   const long long src = rows ? (long long)rows[r] : (long long)r;
@@ -97,7 +100,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restri
   for (int j = threadIdx.x; j < H; j += NT) {
     float v = x[j];
     if (d) {
-      v += delta_sum(d + j, parts, part_stride, round_parts);
+      v += delta_scale * delta_sum(d + j, parts, part_stride, round_parts);
       if (write_resid) x[j] = v;
     }
     ss += v * v;
@@ -108,7 +111,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TD* __restri
   const bool reread_sum = d && !write_resid;
   for (int j = threadIdx.x; j < H; j += NT) {
     float v = x[j];
-    if (reread_sum) v += delta_sum(d + j, parts, part_stride, round_parts);
+    if (reread_sum) v += delta_scale * delta_sum(d + j, parts, part_stride, round_parts);
     st(o + j, v * inv * ld(weight + j));
   }
 }
@@ -119,7 +122,7 @@ template <typename TD, typename TW, typename TO, int NT, int VPT>
 __global__ __launch_bounds__(NT) void add_rmsnorm_small_kernel(
     float* __restrict__ resid, const TD* __restrict__ delta, const TW* __restrict__ weight,
     TO* __restrict__ out, const int* __restrict__ rows, int H, float eps, int write_resid,
-    int parts, long long part_stride, int round_parts) {
+    int parts, long long part_stride, int round_parts, float delta_scale) {
   __shared__ float red[NT / kWave];
   const int r = blockIdx.x;
   const long long src = rows ? (long long)rows[r] : (long long)r;
@@ -134,7 +137,7 @@ __global__ __launch_bounds__(NT) void add_rmsnorm_small_kernel(
     w[i] = 0.f;
     if (j < H) {
       v[i] = x[j];
-      if (d) v[i] += delta_sum(d + j, parts, part_stride, round_parts);
+      if (d) v[i] += delta_scale * delta_sum(d + j, parts, part_stride, round_parts);
       w[i] = ld(weight + j);
     }
     ss += v[i] * v[i];
@@ -343,38 +346,42 @@ template <typename TD, typename TW, typename TO>
 static void launch_add_rmsnorm(float* resid, const void* delta, const void* weight, void* out,
                                const int* rows, int R, int H, float eps, int write_resid,
                                int parts, long long part_stride, int round_parts,
-                               hipStream_t stream) {
+                               float delta_scale, hipStream_t stream) {
   if (H <= 256 * 4)
     add_rmsnorm_small_kernel<TD, TW, TO, 256, 4><<<R, 256, 0, stream>>>(
         resid, (const TD*)delta, (const TW*)weight, (TO*)out, rows, H, eps, write_resid, parts,
-        part_stride, round_parts);
+        part_stride, round_parts, delta_scale);
   else if (H <= 256 * 16)
     add_rmsnorm_small_kernel<TD, TW, TO, 256, 16><<<R, 256, 0, stream>>>(
         resid, (const TD*)delta, (const TW*)weight, (TO*)out, rows, H, eps, write_resid, parts,
-        part_stride, round_parts);
+        part_stride, round_parts, delta_scale);
   else
     add_rmsnorm_kernel<TD, TW, TO, 256><<<R, 256, 0, stream>>>(
         resid, (const TD*)delta, (const TW*)weight, (TO*)out, rows, H, eps, write_resid, parts,
-        part_stride, round_parts);
+        part_stride, round_parts, delta_scale);
 }
 
 RLIS_API int rlis_add_rmsnorm(float* resid, const void* delta, int delta_dtype,
                               const void* weight, int weight_dtype, void* out, int out_dtype,
                               const int* rows, int R, int H, float eps, int write_resid,
                               int parts, long long part_stride, int round_parts,
-                              hipStream_t stream) {
+                              float delta_scale, hipStream_t stream) {
   RLIS_REQUIRE(R >= 0 && H > 0, "add_rmsnorm: bad sizes R=%d H=%d", R, H);
   RLIS_REQUIRE(parts >= 1, "add_rmsnorm: parts=%d", parts);
   RLIS_REQUIRE(!(rows && write_resid && delta),
                "add_rmsnorm: writing the residual back needs all rows, not a selection");
   if (R == 0) return 0;
-  if ((!delta || delta_dtype == RLIS_BF16) && weight_dtype == RLIS_BF16 && out_dtype == RLIS_BF16 &&
+  // (the forms below for special layouts add the delta as it is; a delta that comes with a
+  // multiplier takes the general kernels)
+  const bool plain_delta = !delta || delta_scale == 1.0f;
+  if (plain_delta && (!delta || delta_dtype == RLIS_BF16) && weight_dtype == RLIS_BF16 &&
+      out_dtype == RLIS_BF16 &&
       launch_add_rmsnorm_bf16x8(resid, delta, weight, out, rows, R, H, eps, write_resid, parts,
                                 stream)) {
     RLIS_LAUNCH_CHECK("add_rmsnorm");
     return 0;
   }
-  if (delta && delta_dtype == RLIS_F32 && parts > 1) {
+  if (plain_delta && delta && delta_dtype == RLIS_F32 && parts > 1) {
     bool took = false;
     if (weight_dtype == RLIS_BF16 && out_dtype == RLIS_BF16)
       took = launch_add_rmsnorm_stack<bf16_t, bf16_t>(resid, delta, weight, out, rows, R, H, eps,
@@ -397,7 +404,7 @@ RLIS_API int rlis_add_rmsnorm(float* resid, const void* delta, int delta_dtype,
 #define CASE(k, TD, TW, TO)                                                                  \
   case k:                                                                                    \
     launch_add_rmsnorm<TD, TW, TO>(resid, delta, weight, out, rows, R, H, eps, write_resid,  \
-                                   parts, part_stride, round_parts, stream);                 \
+                                   parts, part_stride, round_parts, delta_scale, stream);    \
     break;
   switch (key) {
     CASE(0, float, float, float)
@@ -482,6 +489,100 @@ RLIS_API int rlis_swiglu(void* out, const void* gu, int dtype, int T, int I, hip
   else
     RLIS_REQUIRE(false, "swiglu: unknown dtype %d", dtype);
   RLIS_LAUNCH_CHECK("swiglu");
+  return 0;
+}
+
+// ------------------------------------------------------------- clamped gated unit
+// gu (T, 2I) as above.  g = min(gate, limit), u = clamp(up, -limit, limit),
+// y = g * sigmoid(alpha * g) * (u + 1): a gated unit whose two branches are bounded before
+// they meet.  float32 arithmetic, one rounding at the store.
+template <typename TX>
+__global__ void clamped_glu_kernel(TX* __restrict__ out, const TX* __restrict__ gu, int I,
+                                   long long total, float limit, float alpha) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (; i < total; i += stride) {
+    const long long t = i / I;
+    const int c = (int)(i - t * I);
+    const float g = fminf(ld(gu + t * 2 * I + c), limit);
+    const float u = fminf(fmaxf(ld(gu + t * 2 * I + I + c), -limit), limit);
+    st(out + i, g / (1.0f + expf(-alpha * g)) * (u + 1.0f));
+  }
+}
+
+RLIS_API int rlis_clamped_glu(void* out, const void* gu, int dtype, int T, int I, float limit,
+                              float alpha, hipStream_t stream) {
+  RLIS_REQUIRE(T >= 0 && I > 0, "clamped_glu: bad sizes T=%d I=%d", T, I);
+  const long long total = (long long)T * I;
+  if (total == 0) return 0;
+  const int blocks = (int)(ceil_div_ll(total, 256) < 8192 ? ceil_div_ll(total, 256) : 8192);
+  if (dtype == RLIS_F32)
+    clamped_glu_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, (const float*)gu, I, total,
+                                                          limit, alpha);
+  else if (dtype == RLIS_BF16)
+    clamped_glu_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)gu, I,
+                                                           total, limit, alpha);
+  else
+    RLIS_REQUIRE(false, "clamped_glu: unknown dtype %d", dtype);
+  RLIS_LAUNCH_CHECK("clamped_glu");
+  return 0;
+}
+
+// ------------------------------------------------------------- weighted sum of two
+// out (float32) = a * x + b * y, element by element: two branches that read the same input
+// meet here on their way into the residual stream.
+template <typename TX, typename TY>
+__global__ void weighted_sum_kernel(float* __restrict__ out, const TX* __restrict__ x, float a,
+                                    const TY* __restrict__ y, float b, long long n) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) out[i] = a * ld(x + i) + b * ld(y + i);
+}
+
+RLIS_API int rlis_weighted_sum(float* out, const void* x, int x_dtype, float a, const void* y,
+                               int y_dtype, float b, long long n, hipStream_t stream) {
+  if (n <= 0) return 0;
+  const int blocks = (int)(ceil_div_ll(n, 256) < 8192 ? ceil_div_ll(n, 256) : 8192);
+  const int key = x_dtype * 2 + y_dtype;
+#define CASE(k, TX, TY)                                                                       \
+  case k:                                                                                     \
+    weighted_sum_kernel<TX, TY><<<blocks, 256, 0, stream>>>(out, (const TX*)x, a, (const TY*)y, \
+                                                            b, n);                            \
+    break;
+  switch (key) {
+    CASE(0, float, float)
+    CASE(1, float, bf16_t)
+    CASE(2, bf16_t, float)
+    CASE(3, bf16_t, bf16_t)
+    default:
+      RLIS_REQUIRE(false, "weighted_sum: unknown dtypes %d %d", x_dtype, y_dtype);
+  }
+#undef CASE
+  RLIS_LAUNCH_CHECK("weighted_sum");
+  return 0;
+}
+
+// ------------------------------------------------------------- tanh, in place
+// x <- cap * tanh(x / cap) (cap 1: the plain function): the bound on the logits, and the
+// activation between the two thin products of a low-rank projection.
+template <typename TX>
+__global__ void soft_cap_kernel(TX* __restrict__ x, long long n, float cap, float inv_cap) {
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) st(x + i, cap * tanhf(ld(x + i) * inv_cap));
+}
+
+RLIS_API int rlis_soft_cap(void* x, int dtype, long long n, float cap, hipStream_t stream) {
+  RLIS_REQUIRE(cap > 0.f, "soft_cap: the cap must be positive");
+  if (n <= 0) return 0;
+  const int blocks = (int)(ceil_div_ll(n, 256) < 8192 ? ceil_div_ll(n, 256) : 8192);
+  if (dtype == RLIS_F32)
+    soft_cap_kernel<float><<<blocks, 256, 0, stream>>>((float*)x, n, cap, 1.0f / cap);
+  else if (dtype == RLIS_BF16)
+    soft_cap_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)x, n, cap, 1.0f / cap);
+  else
+    RLIS_REQUIRE(false, "soft_cap: unknown dtype %d", dtype);
+  RLIS_LAUNCH_CHECK("soft_cap");
   return 0;
 }
 

@@ -53,6 +53,11 @@ def load_model(folder: str, dtype: Union[str, torch.dtype], max_positions: int,
     cfg_dict = read_config_dict(folder)
     arch = architecture_of(cfg_dict)
     cfg = arch.parse_config(cfg_dict)
+    if arch.complete_config is not None:
+        # sizes that the design leaves to the tensors' shapes
+        from ..weights.safetensors_io import open_folder
+        shapes = {name: tuple(f.info(name)[1]) for f in open_folder(folder) for name in f.names()}
+        cfg = arch.complete_config(cfg, shapes)
     spec = arch.build_spec(cfg)
     weights = load_weights(folder, spec.tensor_specs(), act, device, spec.optional_tensors)
     limit = getattr(cfg, "max_position_embeddings", max_positions)

@@ -172,15 +172,15 @@ def _i32(t: torch.Tensor, name: str, n: Optional[int] = None) -> int:
 
 
 # --------------------------------------------------------------------------- rows
-def embed(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
-    """Rows ``table[ids]`` as the float32 residual stream ``(T, H)``."""
+def embed(ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """Rows ``table[ids] * scale`` as the float32 residual stream ``(T, H)``."""
     _check(table, "embed table", ndim=2)
     T, (V, H) = ids.numel(), table.shape
     if not table.is_contiguous():
         raise KernelError("embed table must be contiguous")
     out = torch.empty((T, H), dtype=torch.float32, device=table.device)
     lib.call("rlis_embed", out.data_ptr(), table.data_ptr(), _dt(table), _i32(ids, "ids", T),
-             T, H, lib.stream_ptr())
+             T, H, float(scale), lib.stream_ptr())
     return out
 
 
@@ -199,22 +199,26 @@ def _delta_parts(resid: torch.Tensor, delta: torch.Tensor, what: str) -> int:
                       f"{tuple(resid.shape)}")
 
 
-def add_residual(resid: torch.Tensor, delta: torch.Tensor, round_parts: bool = False) -> None:
-    """``resid += delta`` with the sum formed in float32.  ``round_parts``: a stack of partial
-    sums (of one slice or of many) is added up and rounded to bfloat16 before it joins the
-    residual."""
+def add_residual(resid: torch.Tensor, delta: torch.Tensor, round_parts: bool = False,
+                 delta_scale: float = 1.0) -> None:
+    """``resid += delta_scale * delta`` with product and sum formed in float32.  ``round_parts``:
+    a stack of partial sums (of one slice or of many) is added up and rounded to bfloat16 before
+    it joins the residual."""
     _check(resid, "residual", torch.float32)
     if not resid.is_contiguous():
         raise KernelError("add_residual: residual must be contiguous")
     parts = _delta_parts(resid, delta, "add_residual")
     lib.call("rlis_add_residual", resid.data_ptr(), delta.data_ptr(), _dt(delta), resid.numel(),
-             parts, int(bool(round_parts) and delta.dim() > resid.dim()), lib.stream_ptr())
+             parts, int(bool(round_parts) and delta.dim() > resid.dim()), float(delta_scale),
+             lib.stream_ptr())
 
 
 def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor,
                 eps: float, out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None,
-                write_resid: bool = True, round_parts: bool = False) -> torch.Tensor:
-    """``norm(resid + delta) * weight`` row by row (``round_parts`` as in ``add_residual``).
+                write_resid: bool = True, round_parts: bool = False,
+                delta_scale: float = 1.0) -> torch.Tensor:
+    """``norm(resid + delta_scale * delta) * weight`` row by row (``round_parts`` as in
+    ``add_residual``).
 
     With ``rows`` only those rows are produced and the residual is left as it is; otherwise
     the sum is stored back into ``resid`` when ``write_resid`` is set."""
@@ -236,7 +240,7 @@ def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torc
              weight.data_ptr(), _dt(weight), out.data_ptr(), _DT[out_dtype], rows_ptr, R, H,
              float(eps), int(bool(write_resid)), parts, T * H,
              int(bool(round_parts) and delta is not None and delta.dim() > resid.dim()),
-             lib.stream_ptr())
+             float(delta_scale), lib.stream_ptr())
     return out
 
 
@@ -250,6 +254,43 @@ def swiglu(gu: torch.Tensor) -> torch.Tensor:
     lib.call("rlis_swiglu", out.data_ptr(), gu.data_ptr(), _dt(gu), T, two_i // 2,
              lib.stream_ptr())
     return out
+
+
+def clamped_glu(gu: torch.Tensor, limit: float, alpha: float) -> torch.Tensor:
+    """For ``gu = [gate | up]`` of shape ``(T, 2 I)``: ``g * sigmoid(alpha * g) * (u + 1)`` with
+    ``g = min(gate, limit)`` and ``u = clamp(up, -limit, limit)``."""
+    _check(gu, "gate/up", ndim=2)
+    T, two_i = gu.shape
+    if two_i % 2 or not gu.is_contiguous():
+        raise KernelError("clamped_glu: input must be contiguous with an even number of columns")
+    out = torch.empty((T, two_i // 2), dtype=gu.dtype, device=gu.device)
+    lib.call("rlis_clamped_glu", out.data_ptr(), gu.data_ptr(), _dt(gu), T, two_i // 2,
+             float(limit), float(alpha), lib.stream_ptr())
+    return out
+
+
+def weighted_sum(x: torch.Tensor, a: float, y: torch.Tensor, b: float) -> torch.Tensor:
+    """``a * x + b * y`` in float32, for two tensors of one shape (float32 or bfloat16 each)."""
+    _check(x, "weighted_sum x")
+    _check(y, "weighted_sum y")
+    if x.shape != y.shape or not x.is_contiguous() or not y.is_contiguous():
+        raise KernelError(f"weighted_sum: contiguous tensors of one shape, got {tuple(x.shape)} "
+                          f"and {tuple(y.shape)}")
+    out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    lib.call("rlis_weighted_sum", out.data_ptr(), x.data_ptr(), _dt(x), float(a), y.data_ptr(),
+             _dt(y), float(b), x.numel(), lib.stream_ptr())
+    return out
+
+
+def soft_cap_(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """``x <- cap * tanh(x / cap)`` in place (``cap`` 1: the plain tanh)."""
+    _check(x, "soft_cap")
+    if not x.is_contiguous():
+        raise KernelError("soft_cap: tensor must be contiguous")
+    if not cap > 0:
+        raise KernelError("soft_cap: the cap must be positive")
+    lib.call("rlis_soft_cap", x.data_ptr(), _dt(x), x.numel(), float(cap), lib.stream_ptr())
+    return x
 
 
 # ----------------------------------------------------------------------- products
@@ -972,6 +1013,10 @@ def sample_rows(logits: torch.Tensor, keys: torch.Tensor, inv_temps: torch.Tenso
              None if best is None else best.data_ptr(), None if idx is None else idx.data_ptr(),
              lib.stream_ptr())
     return out
+
+
+from .recurrent import (causal_conv, decay_scan, delta_scan, head_norm_gate,  # noqa: E402,F401
+                        shift_mix, tail_update)
 
 
 def fill_normal(out: torch.Tensor, seed: int, tensor_index: int, mean: float, std: float) -> None:

@@ -17,10 +17,19 @@ _LIB: Optional[ctypes.CDLL] = None
 P, I, L, F = c_void_p, c_int, c_longlong, c_float
 
 _SIGNATURES = {
-    "rlis_embed": [P, P, I, P, I, I, P],
-    "rlis_add_residual": [P, P, I, L, I, I, P],
-    "rlis_add_rmsnorm": [P, P, I, P, I, P, I, P, I, I, F, I, I, L, I, P],
+    "rlis_embed": [P, P, I, P, I, I, F, P],
+    "rlis_add_residual": [P, P, I, L, I, I, F, P],
+    "rlis_add_rmsnorm": [P, P, I, P, I, P, I, P, I, I, F, I, I, L, I, F, P],
     "rlis_swiglu": [P, P, I, I, I, P],
+    "rlis_clamped_glu": [P, P, I, I, I, F, F, P],
+    "rlis_weighted_sum": [P, P, I, F, P, I, F, L, P],
+    "rlis_soft_cap": [P, I, L, F, P],
+    "rlis_shift_mix": [P, P, I, P, P, L, P, P, P, I, I, I, P],
+    "rlis_tail_update": [P, L, P, I, L, I, I, P, P, I, P],
+    "rlis_causal_conv": [P, P, L, P, I, I, P, L, P, P, P, I, I, I, I, F, F, I, P],
+    "rlis_delta_scan": [P, L, P, P, P, L, P, P, L, P, P, P, L, P, P, I, I, I, I, I, P],
+    "rlis_decay_scan": [P, P, P, P, P, L, P, P, P, L, P, P, I, I, I, P],
+    "rlis_head_norm_gate": [P, I, P, P, I, P, I, L, I, I, I, F, P],
     "rlis_rope_kv_write": [P, I, L, I, I, I, I, I, I, I, P, P, P, P, P, P, I, I, I, I, P],
     "rlis_copy_pages": [P, I, I, L, L, P, P, I, P],
     "rlis_gemm_plain": [P, I, P, I, P, I, I, I, I, L, L, L, P],

@@ -1,0 +1,191 @@
+"""The kernels of mixers with a state of fixed size per request (``csrc/kernels/recurrent.hip``)
+as Python functions: token shift, input tails, the short causal convolution, the two scans over
+a matrix state per head, and the per-head norm with weight and gate behind them.
+
+A ``state`` argument is a float32 view ``(slots, n)`` of the mixer's area in the runner's state
+buffer (rows a whole slot apart); ``cu``, ``slots`` and ``seq_of_token`` are the step's
+cumulative token counts, state slots and sequence of each token, int32 on the device.  Every
+function checks on the host what its kernel and grid assume."""
+from __future__ import annotations
+
+import torch
+
+from . import lib
+from .lib import KernelError
+
+_DT = {torch.float32: 0, torch.bfloat16: 1}
+
+
+def _dt(t: torch.Tensor) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise KernelError(f"unsupported dtype {t.dtype} (float32 and bfloat16 only)") from None
+
+
+def _state(state: torch.Tensor, need: int, what: str) -> int:
+    if not state.is_cuda or state.dtype != torch.float32 or state.dim() != 2:
+        raise KernelError(f"{what}: the state must be a float32 (slots, n) view on the GPU")
+    if state.shape[1] < need or (state.shape[1] > 1 and state.stride(1) != 1):
+        raise KernelError(f"{what}: the state holds {state.shape[1]} floats a slot, {need} needed")
+    return state.stride(0) if state.shape[0] > 1 else max(state.stride(0), state.shape[1])
+
+
+def _meta(t: torch.Tensor, n: int, what: str) -> int:
+    if not t.is_cuda or t.dtype != torch.int32 or not t.is_contiguous() or t.numel() < n:
+        raise KernelError(f"{what}: needs {n} contiguous int32 entries on the GPU")
+    return t.data_ptr()
+
+
+def _rows(t: torch.Tensor, what: str, dtype=None) -> int:
+    """Row stride of a 2-D tensor whose rows are contiguous."""
+    if not t.is_cuda or t.dim() != 2 or (t.shape[1] > 1 and t.stride(1) != 1):
+        raise KernelError(f"{what}: a 2-D tensor on the GPU with contiguous rows is needed")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{what}: expected {dtype}, got {t.dtype}")
+    return t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+
+
+def _vec(t: torch.Tensor, n: int, what: str) -> int:
+    if not t.is_cuda or t.dtype != torch.float32 or not t.is_contiguous() or t.numel() != n:
+        raise KernelError(f"{what}: needs {n} contiguous float32 values on the GPU, got "
+                          f"{tuple(t.shape)} {t.dtype}")
+    return t.data_ptr()
+
+
+def shift_mix(x: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, seq_of_token: torch.Tensor,
+              cu: torch.Tensor, slots: torch.Tensor, num_seqs: int) -> torch.Tensor:
+    """``out[m] = x + (prev - x) * mu[m]`` for every row of ``x (T, W)``, ``prev`` being the row
+    of the token before (for a sequence's first token of the step: the row kept in ``state``).
+    Returns ``(mixes, T, W)`` in the dtype of ``x``."""
+    if not x.is_cuda or x.dim() != 2 or not x.is_contiguous():
+        raise KernelError("shift_mix: x must be a contiguous (T, W) tensor on the GPU")
+    T, W = x.shape
+    mixes = mu.shape[0]
+    _vec(mu.reshape(-1), mixes * W, "shift_mix mu")
+    stride = _state(state, W, "shift_mix")
+    out = torch.empty((mixes, T, W), dtype=x.dtype, device=x.device)
+    lib.call("rlis_shift_mix", out.data_ptr(), x.data_ptr(), _dt(x), mu.data_ptr(),
+             state.data_ptr(), stride, _meta(seq_of_token, T, "seq_of_token"),
+             _meta(cu, num_seqs + 1, "cu"), _meta(slots, num_seqs, "slots"), T, W, mixes,
+             lib.stream_ptr())
+    return out
+
+
+def tail_update(state: torch.Tensor, x: torch.Tensor, channels: int, rows: int, cu: torch.Tensor,
+                slots: torch.Tensor, num_seqs: int) -> None:
+    """Every sequence's tail in ``state`` (``rows`` rows of ``channels`` floats, oldest first)
+    becomes the last ``rows`` of (its old tail, then the step's rows of ``x[:, :channels]``)."""
+    ldx = _rows(x, "tail_update x")
+    if x.shape[1] < channels:
+        raise KernelError(f"tail_update: x has {x.shape[1]} columns, {channels} needed")
+    stride = _state(state, channels * rows, "tail_update")
+    lib.call("rlis_tail_update", state.data_ptr(), stride, x.data_ptr(), _dt(x), ldx, channels,
+             rows, _meta(cu, num_seqs + 1, "cu"), _meta(slots, num_seqs, "slots"), num_seqs,
+             lib.stream_ptr())
+
+
+def causal_conv(x: torch.Tensor, taps: torch.Tensor, state: torch.Tensor,
+                seq_of_token: torch.Tensor, cu: torch.Tensor, slots: torch.Tensor, num_seqs: int,
+                unit_channels: int = 0, unit_group: int = 0, scaled_channels: int = 0,
+                scale: float = 1.0, unit_eps: float = 0.0, rest_group: int = 256) -> torch.Tensor:
+    """``silu`` of the causal convolution over time of the first ``C`` columns of ``x`` (float32)
+    with ``taps (C, K)`` (the last column multiplies the current row; the ``K - 1`` rows in
+    front of the step come from ``state``).  Channels below ``unit_channels`` are then made
+    unit vectors in groups of ``unit_group``: ``y / sqrt(sum y^2 + unit_eps)``, those below
+    ``scaled_channels`` times ``scale``.  Returns ``(T, C)`` float32."""
+    ldx = _rows(x, "causal_conv x", torch.float32)
+    C, K = taps.shape
+    _vec(taps.reshape(-1), C * K, "causal_conv taps")
+    if x.shape[1] < C:
+        raise KernelError(f"causal_conv: x has {x.shape[1]} columns, the taps {C} channels")
+    T = x.shape[0]
+    stride = _state(state, C * (K - 1), "causal_conv")
+    out = torch.empty((T, C), dtype=torch.float32, device=x.device)
+    lib.call("rlis_causal_conv", out.data_ptr(), x.data_ptr(), ldx, taps.data_ptr(), C, K,
+             state.data_ptr(), stride, _meta(seq_of_token, T, "seq_of_token"),
+             _meta(cu, num_seqs + 1, "cu"), _meta(slots, num_seqs, "slots"), T,
+             int(unit_channels), int(unit_group), int(scaled_channels), float(scale),
+             float(unit_eps), int(rest_group), lib.stream_ptr())
+    return out
+
+
+def delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, b_raw: torch.Tensor,
+               a_raw: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor,
+               state: torch.Tensor, cu: torch.Tensor, slots: torch.Tensor, num_seqs: int,
+               heads: int, kv_heads: int, dk: int, dv: int) -> torch.Tensor:
+    """The gated delta rule over every sequence's tokens of the step.  ``q``, ``k``
+    ``(T, kv_heads * dk)`` and ``v (T, heads * dv)`` are float32 column ranges of one matrix
+    (one row stride), ``b_raw``, ``a_raw`` ``(T, heads)`` of another; per token and head
+    ``S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q`` with
+    ``g = exp(-exp(a_log) * softplus(a_raw + dt_bias))`` and ``beta = sigmoid(b_raw)``.
+    ``state (slots, heads * dv * dk)`` holds S as [head][value channel][key channel] and is
+    left as after each sequence's last token.  Returns ``o (T, heads * dv)`` float32."""
+    ld = _rows(q, "delta_scan q", torch.float32)
+    if _rows(k, "delta_scan k", torch.float32) != ld or _rows(v, "delta_scan v", torch.float32) != ld:
+        raise KernelError("delta_scan: q, k and v must share a row stride")
+    ldba = _rows(b_raw, "delta_scan b", torch.float32)
+    if _rows(a_raw, "delta_scan a", torch.float32) != ldba:
+        raise KernelError("delta_scan: a and b must share a row stride")
+    T = q.shape[0]
+    if q.shape[1] != kv_heads * dk or k.shape != q.shape or v.shape != (T, heads * dv) \
+            or b_raw.shape != (T, heads) or a_raw.shape != (T, heads):
+        raise KernelError("delta_scan: operand shapes do not match the head counts and sizes")
+    stride = _state(state, heads * dv * dk, "delta_scan")
+    out = torch.empty((T, heads * dv), dtype=torch.float32, device=q.device)
+    lib.call("rlis_delta_scan", out.data_ptr(), heads * dv, q.data_ptr(), k.data_ptr(),
+             v.data_ptr(), ld, b_raw.data_ptr(), a_raw.data_ptr(), ldba,
+             _vec(a_log, heads, "delta_scan A_log"), _vec(dt_bias, heads, "delta_scan dt_bias"),
+             state.data_ptr(), stride, _meta(cu, num_seqs + 1, "cu"),
+             _meta(slots, num_seqs, "slots"), num_seqs, heads, kv_heads, dk, dv, lib.stream_ptr())
+    return out
+
+
+def decay_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch.Tensor,
+               w0: torch.Tensor, bonus: torch.Tensor, state: torch.Tensor, cu: torch.Tensor,
+               slots: torch.Tensor, num_seqs: int, heads: int, d: int) -> torch.Tensor:
+    """A matrix state per head with a decay per key channel and a bonus for the current token:
+    per token ``o = (S + diag(bonus) k v^T)^T r; S <- diag(w) S + k v^T`` with
+    ``w = exp(-exp(z + w0))``.  ``r``, ``k``, ``v``, ``z`` are contiguous float32
+    ``(T, heads * d)``; ``state (slots, heads * d * d)`` holds S as [head][value channel][key
+    channel].  Returns ``o (T, heads * d)`` float32."""
+    T = r.shape[0]
+    for name, t in (("r", r), ("k", k), ("v", v), ("z", z)):
+        if not t.is_cuda or t.dtype != torch.float32 or t.shape != (T, heads * d) \
+                or not t.is_contiguous():
+            raise KernelError(f"decay_scan: {name} must be contiguous float32 (T, heads * d)")
+    stride = _state(state, heads * d * d, "decay_scan")
+    out = torch.empty((T, heads * d), dtype=torch.float32, device=r.device)
+    lib.call("rlis_decay_scan", out.data_ptr(), r.data_ptr(), k.data_ptr(), v.data_ptr(),
+             z.data_ptr(), heads * d, _vec(w0, heads * d, "decay_scan w0"),
+             _vec(bonus.reshape(-1), heads * d, "decay_scan bonus"), state.data_ptr(), stride,
+             _meta(cu, num_seqs + 1, "cu"), _meta(slots, num_seqs, "slots"), num_seqs, heads, d,
+             lib.stream_ptr())
+    return out
+
+
+def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, heads: int, dv: int,
+                   eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """``o / sqrt(mean o^2 + eps)`` per head, times ``weight`` (``heads * dv`` values, or ``dv``
+    shared by the heads), times ``silu(gate)``.  ``o`` contiguous float32 ``(T, heads * dv)``,
+    ``gate`` of that shape with contiguous rows."""
+    T = o.shape[0]
+    if not o.is_cuda or o.dtype != torch.float32 or o.shape != (T, heads * dv) \
+            or not o.is_contiguous():
+        raise KernelError("head_norm_gate: o must be contiguous float32 (T, heads * dv)")
+    ldg = _rows(gate, "head_norm_gate gate")
+    if gate.shape != o.shape:
+        raise KernelError("head_norm_gate: the gate must have the shape of o")
+    if weight.numel() == heads * dv and heads > 1:
+        wstride = dv
+    elif weight.numel() == dv:
+        wstride = 0
+    else:
+        raise KernelError(f"head_norm_gate: weight of {weight.numel()} values for {heads} heads "
+                          f"of {dv}")
+    _vec(weight.reshape(-1), weight.numel(), "head_norm_gate weight")
+    out = torch.empty((T, heads * dv), dtype=out_dtype, device=o.device)
+    lib.call("rlis_head_norm_gate", out.data_ptr(), _DT[out_dtype], o.data_ptr(),
+             weight.data_ptr(), wstride, gate.data_ptr(), _dt(gate), ldg, T, heads, dv, float(eps),
+             lib.stream_ptr())
+    return out

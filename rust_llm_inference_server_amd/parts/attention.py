@@ -22,7 +22,17 @@ from .rope import shared_position
 @register("mixer", "attention")
 class PagedAttention(Mixer):
     """Parameters: ``hidden_size``, ``num_heads``, ``num_kv_heads``, ``head_dim``, ``scale``,
-    ``window`` (None: all earlier positions), ``position`` (a PartSpec).
+    ``window`` (None: all earlier positions), ``position`` (a PartSpec); optional ``value_dim``
+    (size of a value head when it differs from ``head_dim``, the size of a query and key head)
+    and ``names`` (the tensors of q, k, v and o under the prefix; default ``q_proj.weight`` and
+    so on).
+
+    With ``value_dim != head_dim`` the kernels run at one head size ``D``, the larger of the two
+    rounded up to a multiple of 16: the rows of the narrower projection's weight are padded
+    with zero rows per head at build time (and the output projection's columns with zero
+    columns), so the extra query and key dims add exact zeros to every score and the extra
+    value dims come out as exact zeros that meet zero columns.  The kernels stay specialised on
+    one head size; the price is that the narrower of keys and values is cached at ``D``.
 
     What the position part may carry: ``rot_dim``, ``cos``, ``sin`` (float32 tables, a rotation
     of the first ``rot_dim`` dims of every q and k head; rot_dim 0: none), ``interleaved``
@@ -34,34 +44,61 @@ class PagedAttention(Mixer):
     takes_normed_input = True
 
     @classmethod
+    def _names(cls, params: Dict[str, Any], prefix: str) -> Dict[str, str]:
+        names = {**{n: f"{n}_proj.weight" for n in "qkvo"}, **(params.get("names") or {})}
+        return {k: join(prefix, v) for k, v in names.items()}
+
+    @classmethod
     def tensor_specs(cls, params: Dict[str, Any], prefix: str) -> List[TensorSpec]:
         H, nh, nkv, d = (params[k] for k in ("hidden_size", "num_heads", "num_kv_heads",
                                              "head_dim"))
-        return [TensorSpec(join(prefix, "q_proj.weight"), (nh * d, H)),
-                TensorSpec(join(prefix, "k_proj.weight"), (nkv * d, H)),
-                TensorSpec(join(prefix, "v_proj.weight"), (nkv * d, H)),
-                TensorSpec(join(prefix, "o_proj.weight"), (H, nh * d))]
+        dv = params.get("value_dim") or d
+        n = cls._names(params, prefix)
+        return [TensorSpec(n["q"], (nh * d, H)), TensorSpec(n["k"], (nkv * d, H)),
+                TensorSpec(n["v"], (nkv * dv, H)), TensorSpec(n["o"], (H, nh * dv))]
+
+    @staticmethod
+    def _pad_heads(w: torch.Tensor, heads: int, size: int, to: int, rows: bool) -> torch.Tensor:
+        """A projection whose heads of ``size`` lie along its rows (or columns) with every head
+        padded to ``to`` by zeros."""
+        if size == to:
+            return w
+        if rows:
+            out = w.new_zeros((heads, to, w.shape[1]))
+            out[:, :size] = w.reshape(heads, size, w.shape[1])
+            return out.reshape(heads * to, w.shape[1])
+        out = w.new_zeros((w.shape[0], heads, to))
+        out[:, :, :size] = w.reshape(w.shape[0], heads, size)
+        return out.reshape(w.shape[0], heads * to)
 
     def __init__(self, params: Dict[str, Any], prefix: str, ctx: BuildContext):
         super().__init__(params, prefix, ctx)
         self.num_heads = int(params["num_heads"])
         self.num_kv_heads = int(params["num_kv_heads"])
-        self.head_dim = int(params["head_dim"])
+        qk_dim = int(params["head_dim"])
+        v_dim = int(params.get("value_dim") or qk_dim)
+        # the one head size the kernels run at
+        self.head_dim = qk_dim if v_dim == qk_dim else -(-max(qk_dim, v_dim) // 16) * 16
         self.scale = float(params["scale"])
         self.window: Optional[int] = params.get("window")
         if self.num_heads % self.num_kv_heads:
             raise ValueError(f"attention: {self.num_heads} heads are not a multiple of "
                              f"{self.num_kv_heads} KV heads")
-        q, k, v = (ctx.weights.pop(join(prefix, f"{n}_proj.weight")) for n in "qkv")
+        names = self._names(params, prefix)
+        q, k, v = (ctx.weights.pop(names[n]) for n in "qkv")
         if not (q.dtype == k.dtype == v.dtype):
             q, k, v = (t.to(torch.float32) for t in (q, k, v))
+        q = self._pad_heads(q, self.num_heads, qk_dim, self.head_dim, rows=True)
+        k = self._pad_heads(k, self.num_kv_heads, qk_dim, self.head_dim, rows=True)
+        v = self._pad_heads(v, self.num_kv_heads, v_dim, self.head_dim, rows=True)
         # One product for q, k and v: the rows of the three weights, concatenated.
         self.w_qkv = torch.cat([q, k, v], dim=0).contiguous()
         del q, k, v
-        self.w_o = ctx.take(join(prefix, "o_proj.weight"))
+        self.w_o = self._pad_heads(ctx.take(names["o"]), self.num_heads, v_dim, self.head_dim,
+                                   rows=False).contiguous()
         self.act_dtype = ctx.act_dtype
         self.position = shared_position(params.get("position") or PartSpec("none"), ctx)
-        if self.position.rot_dim > self.head_dim:
+        if self.position.rot_dim > qk_dim:
             raise ValueError("attention: the rotated width exceeds the head size")
 
         self.planner = ops.attention_planner(

@@ -200,6 +200,10 @@ def tensor_specs(category: str, spec: PartSpec, prefix: str) -> List[TensorSpec]
 
 
 def join(prefix: str, name: str) -> str:
+    """``prefix.name``; an empty name is the prefix itself (a part whose one tensor is stored
+    under the part's own name)."""
+    if not name:
+        return prefix
     return f"{prefix}.{name}" if prefix else name
 
 
@@ -370,7 +374,7 @@ class ResidualStream:
     (``round_parts``), as a delta that arrives whole in bfloat16 was by its kernel, so that the
     rounding does not depend on which kernel a batch's size chose."""
 
-    __slots__ = ("x", "pending", "round_parts")
+    __slots__ = ("x", "pending", "pending_scale", "round_parts")
 
     def __init__(self, x: torch.Tensor, act_dtype: torch.dtype = torch.float32):
         assert x.dtype == torch.float32
@@ -378,12 +382,22 @@ class ResidualStream:
         # a tensor, or a product that has not run yet (``ops.pending_linear``), which a norm
         # may run with the add and its own multiplies inside
         self.pending: Any = None
+        # the multiplier with which the pending delta joins the sum (in float32, by whoever
+        # adds it); a norm's fused forms take deltas with multiplier 1 only
+        self.pending_scale = 1.0
         self.round_parts = act_dtype == torch.bfloat16
 
-    def add(self, delta: Any) -> None:
+    def add(self, delta: Any, scale: float = 1.0) -> None:
         if self.pending is not None:
             self.flush()
         self.pending = delta
+        self.pending_scale = float(scale)
+
+    def take_delta(self) -> Tuple[Optional[torch.Tensor], float]:
+        """The pending delta as a tensor with its multiplier; the stream then has none."""
+        delta, scale = self.delta(), self.pending_scale
+        self.pending, self.pending_scale = None, 1.0
+        return delta, scale
 
     def delta(self) -> Optional[torch.Tensor]:
         """The pending delta as a tensor (a product that has not run yet runs now)."""
@@ -395,6 +409,7 @@ class ResidualStream:
         """Fold a pending delta into the residual and return the residual."""
         if self.pending is not None:
             from .. import ops
-            ops.add_residual(self.x, self.delta(), round_parts=self.round_parts)
-            self.pending = None
+            ops.add_residual(self.x, self.delta(), round_parts=self.round_parts,
+                             delta_scale=self.pending_scale)
+            self.pending, self.pending_scale = None, 1.0
         return self.x

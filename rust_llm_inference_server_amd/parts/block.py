@@ -12,31 +12,44 @@ from .base import (Block, BuildContext, CacheBinding, ResidualStream, TensorSpec
 @register("block", "prenorm")
 class PreNormBlock(Block):
     """Parameters: ``mixer``, ``feed_forward``, ``mixer_norm``, ``ffn_norm`` (PartSpecs) and
-    ``names``: the weight-name suffix of each of the four under the block's prefix."""
+    ``names``: the weight-name suffix of each of the four under the block's prefix.  A block
+    whose ``feed_forward`` is None has the mixer's sublayer only.  Optional
+    ``residual_scale`` m: each sublayer's output joins the stream as ``x += m * f(norm(x))``,
+    the product formed in float32 where the sum is."""
 
     _SLOTS = (("mixer_norm", "norm"), ("mixer", "mixer"), ("ffn_norm", "norm"),
               ("feed_forward", "feed_forward"))
 
     @classmethod
+    def _slots(cls, params: Dict[str, Any]):
+        if params.get("feed_forward") is None:
+            return cls._SLOTS[:2]
+        return cls._SLOTS
+
+    @classmethod
     def tensor_specs(cls, params: Dict[str, Any], prefix: str) -> List[TensorSpec]:
         out: List[TensorSpec] = []
-        for slot, category in cls._SLOTS:
+        for slot, category in cls._slots(params):
             out += tensor_specs(category, params[slot], join(prefix, params["names"][slot]))
         return out
 
     def __init__(self, params: Dict[str, Any], prefix: str, ctx: BuildContext):
         super().__init__(params, prefix, ctx)
         built = {slot: create(category, params[slot], join(prefix, params["names"][slot]), ctx)
-                 for slot, category in self._SLOTS}
+                 for slot, category in self._slots(params)}
         self.mixer_norm, self.mixer = built["mixer_norm"], built["mixer"]
-        self.ffn_norm, self.feed_forward = built["ffn_norm"], built["feed_forward"]
+        self.ffn_norm, self.feed_forward = built.get("ffn_norm"), built.get("feed_forward")
+        self.residual_scale = float(params.get("residual_scale", 1.0))
 
     @property
     def graph_safe(self) -> bool:
         return all(p.graph_safe for p in (self.mixer_norm, self.mixer, self.ffn_norm,
-                                          self.feed_forward))
+                                          self.feed_forward) if p is not None)
 
     def forward(self, stream: ResidualStream, step: Any, binding: CacheBinding) -> None:
-        stream.add(self.mixer.forward(normed(self.mixer_norm, stream, self.mixer), step, binding))
-        stream.add(self.feed_forward.forward(normed(self.ffn_norm, stream, self.feed_forward),
-                                             step))
+        m = self.residual_scale
+        stream.add(self.mixer.forward(normed(self.mixer_norm, stream, self.mixer), step, binding),
+                   m)
+        if self.feed_forward is not None:
+            stream.add(self.feed_forward.forward(
+                normed(self.ffn_norm, stream, self.feed_forward), step), m)

@@ -16,27 +16,32 @@ from .base import BuildContext, Embedding, Head, TensorSpec, join, project, regi
 
 @register("embedding", "token")
 class TokenEmbedding(Embedding):
-    """Parameters: ``vocab_size``, ``hidden_size``."""
+    """Parameters: ``vocab_size``, ``hidden_size``; optional ``scale`` (the rows are multiplied
+    by it as they enter the float32 stream) and ``weight_name`` (the table's name under the
+    prefix, "weight" by default; "" when it is stored under the prefix itself)."""
 
     graph_safe = True
 
     @classmethod
     def tensor_specs(cls, params: Dict[str, Any], prefix: str) -> List[TensorSpec]:
-        return [TensorSpec(join(prefix, "weight"), (params["vocab_size"], params["hidden_size"]))]
+        return [TensorSpec(join(prefix, params.get("weight_name", "weight")),
+                           (params["vocab_size"], params["hidden_size"]))]
 
     def __init__(self, params: Dict[str, Any], prefix: str, ctx: BuildContext):
         super().__init__(params, prefix, ctx)
-        self.weight = ctx.take(join(prefix, "weight"))
+        self.weight = ctx.take(join(prefix, params.get("weight_name", "weight")))
         self.vocab_size = int(params["vocab_size"])
+        self.scale = float(params.get("scale", 1.0))
 
     def forward(self, ids: torch.Tensor) -> torch.Tensor:
-        return ops.embed(ids, self.weight)
+        return ops.embed(ids, self.weight, self.scale)
 
 
 @register("head", "linear")
 class LinearHead(Head):
     """Parameters: ``vocab_size``, ``hidden_size``, ``tied_to`` (name of the tensor to share,
-    or None for a weight of its own at ``prefix.weight``)."""
+    or None for a weight of its own at ``prefix.weight``; ``weight_name`` names it otherwise,
+    "" for the prefix itself); optional ``soft_cap`` c: logits become ``c * tanh(logits / c)``."""
 
     graph_safe = True
 
@@ -46,11 +51,18 @@ class LinearHead(Head):
     def tensor_specs(cls, params: Dict[str, Any], prefix: str) -> List[TensorSpec]:
         if params.get("tied_to"):
             return []
-        return [TensorSpec(join(prefix, "weight"), (params["vocab_size"], params["hidden_size"]))]
+        return [TensorSpec(join(prefix, params.get("weight_name", "weight")),
+                           (params["vocab_size"], params["hidden_size"]))]
 
     def __init__(self, params: Dict[str, Any], prefix: str, ctx: BuildContext):
         super().__init__(params, prefix, ctx)
-        self.weight = ctx.take(params.get("tied_to") or join(prefix, "weight"))
+        self.weight = ctx.take(params.get("tied_to")
+                               or join(prefix, params.get("weight_name", "weight")))
+        cap = params.get("soft_cap")
+        self.soft_cap = float(cap) if cap else None
 
     def forward(self, x: Any) -> torch.Tensor:
-        return project(x, self.weight, torch.float32)
+        logits = project(x, self.weight, torch.float32)
+        if self.soft_cap is not None:
+            ops.soft_cap_(logits, self.soft_cap)
+        return logits

@@ -1,5 +1,6 @@
 """RMSNorm: ``y = x * rsqrt(mean(x^2) + eps) * w`` over the hidden axis; the weight multiplies
-directly, not as ``1 + w`` (crates/model/src/layers.rs:103-122, 141-146).  The input is the
+directly, not as ``1 + w`` (crates/model/src/layers.rs:103-122, 141-146), unless the model
+stores its weights around zero (``weight_offset`` 1: ``y = ... * (1 + w)``).  The input is the
 32-bit residual stream; statistics and both multiplies are 32-bit, one rounding at the store."""
 from __future__ import annotations
 
@@ -13,33 +14,49 @@ from .base import BuildContext, Norm, ResidualStream, TensorSpec, join, register
 
 @register("norm", "rmsnorm")
 class RMSNorm(Norm):
-    """Parameters: ``size`` (hidden width), ``eps``."""
+    """Parameters: ``size`` (hidden width), ``eps``; optional ``weight_offset`` (a number added
+    to the stored weight, in float32, once at build time: 1 for weights stored around zero) and
+    ``weight_name`` (the tensor's name under the prefix, "weight" by default; "" when the
+    tensor is stored under the prefix itself)."""
 
     graph_safe = True
 
     @classmethod
+    def _weight_name(cls, params: Dict[str, Any], prefix: str) -> str:
+        return join(prefix, params.get("weight_name", "weight"))
+
+    @classmethod
     def tensor_specs(cls, params: Dict[str, Any], prefix: str) -> List[TensorSpec]:
-        return [TensorSpec(join(prefix, "weight"), (params["size"],), init="ones_normal")]
+        init = "normal" if float(params.get("weight_offset", 0.0)) else "ones_normal"
+        return [TensorSpec(cls._weight_name(params, prefix), (params["size"],), init=init)]
 
     def __init__(self, params: Dict[str, Any], prefix: str, ctx: BuildContext):
         super().__init__(params, prefix, ctx)
         self.eps = float(params["eps"])
-        self.weight = ctx.take(join(prefix, "weight"))
+        self.weight = ctx.take(self._weight_name(params, prefix))
+        offset = float(params.get("weight_offset", 0.0))
+        if offset:
+            self.weight = (self.weight.to(torch.float32) + offset).contiguous()
         self.out_dtype = ctx.act_dtype
 
     def forward(self, stream: ResidualStream) -> torch.Tensor:
-        delta, stream.pending = stream.delta(), None
+        delta, scale = stream.take_delta()
         return ops.add_rmsnorm(stream.x, delta, self.weight, self.eps, self.out_dtype,
-                               round_parts=stream.round_parts)
+                               round_parts=stream.round_parts, delta_scale=scale)
 
     def forward_rows(self, stream: ResidualStream, rows: torch.Tensor) -> torch.Tensor:
         return ops.add_rmsnorm(stream.x, stream.delta(), self.weight, self.eps, self.out_dtype,
-                               rows=rows, round_parts=stream.round_parts)
+                               rows=rows, round_parts=stream.round_parts,
+                               delta_scale=stream.pending_scale)
 
     def fused_linear(self, stream: ResidualStream, w: torch.Tensor, out_dtype: torch.dtype,
                      gated: bool, rows: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
         if self.out_dtype != torch.bfloat16:
             return None
+        if stream.pending is not None and stream.pending_scale != 1.0:
+            if rows is not None:
+                return None
+            stream.flush()          # the fused forms add a delta as it is
         product = stream.pending
         if isinstance(product, ops.PendingProduct) and rows is None \
                 and ops.can_join_norm_linear(product, stream.x, w):

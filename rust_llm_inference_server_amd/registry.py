@@ -6,12 +6,13 @@ in config.json chooses the model everywhere: loader, engine, replay.
 The registry names no architecture itself.  Each architecture registers from its own module
 (``models/llama.py`` does for ``LlamaForCausalLM``); the modules that ship with the package are
 imported, once, at the first lookup."""
+# (models/gipotar.py registers ``Gipotar`` the same way.)
 from __future__ import annotations
 
 import json
 import os
 from dataclasses import dataclass
-from typing import TYPE_CHECKING, Any, Callable, Dict
+from typing import TYPE_CHECKING, Any, Callable, Dict, Optional
 
 from .config.errors import ConfigError
 
@@ -25,6 +26,9 @@ class Architecture:
     parse_config: Callable[[Dict[str, Any]], Any]      # config.json dict -> typed config
     build_spec: Callable[[Any], "ModelSpec"]           # typed config -> model specification
     config_to_dict: Callable[[Any], Dict[str, Any]]    # typed config -> config.json dict
+    # (typed config, checkpoint tensor name -> shape) -> typed config with the sizes filled in
+    # that the design leaves to the tensors' shapes; None: config.json says everything
+    complete_config: Optional[Callable[[Any, Dict[str, Any]], Any]] = None
 
 
 _ARCHITECTURES: Dict[str, Architecture] = {}
@@ -57,7 +61,11 @@ def architecture_names():
 
 
 def architecture_of(config_dict: Dict[str, Any]) -> Architecture:
+    """The architecture a config.json names: ``architectures[0]`` (the Hugging Face key), or
+    for files that name one design only, the string under ``architecture``."""
     archs = config_dict.get("architectures")
+    if archs is None and isinstance(config_dict.get("architecture"), str):
+        return architecture(config_dict["architecture"])
     if not isinstance(archs, list) or not archs or not isinstance(archs[0], str):
         raise ConfigError("config.json: 'architectures' must be a non-empty list of names")
     return architecture(archs[0])
