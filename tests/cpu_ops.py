@@ -12,17 +12,17 @@ from __future__ import annotations
 import torch
 
 
-def embed(ids, table):
-    return table[ids.long()].to(torch.float32)
+def embed(ids, table, scale=1.0):
+    return table[ids.long()].to(torch.float32) * scale
 
 
-def add_residual(resid, delta, round_parts=False):
-    resid += delta.to(torch.float32)
+def add_residual(resid, delta, round_parts=False, delta_scale=1.0):
+    resid += delta_scale * delta.to(torch.float32)
 
 
 def add_rmsnorm(resid, delta, weight, eps, out_dtype, rows=None, write_resid=True,
-                round_parts=False):
-    x = resid if delta is None else resid + delta.to(torch.float32)
+                round_parts=False, delta_scale=1.0):
+    x = resid if delta is None else resid + delta_scale * delta.to(torch.float32)
     if rows is not None:
         x = x[rows.long()]
     elif delta is not None and write_resid:
@@ -35,6 +35,111 @@ def swiglu(gu):
     i = gu.shape[1] // 2
     g, u = gu[:, :i].float(), gu[:, i:].float()
     return (g / (1.0 + torch.exp(-g)) * u).to(gu.dtype)
+
+
+def clamped_glu(gu, limit, alpha):
+    i = gu.shape[1] // 2
+    g = gu[:, :i].float().clamp(max=limit)
+    u = gu[:, i:].float().clamp(min=-limit, max=limit)
+    return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gu.dtype)
+
+
+def weighted_sum(x, a, y, b):
+    return a * x.float() + b * y.float()
+
+
+def soft_cap_(x, cap):
+    x.copy_((cap * torch.tanh(x.float() / cap)).to(x.dtype))
+    return x
+
+
+# ---- mixers with a state of fixed size: the kernels' contracts, sequence by sequence --------
+def _seqs(cu, slots, num_seqs):
+    cu, slots = cu.tolist(), slots.tolist()
+    return [(cu[s], cu[s + 1], slots[s]) for s in range(num_seqs)]
+
+
+def shift_mix(x, mu, state, seq_of_token, cu, slots, num_seqs):
+    out = torch.empty((mu.shape[0],) + tuple(x.shape), dtype=x.dtype)
+    xf = x.float()
+    for t0, t1, slot in _seqs(cu, slots, num_seqs):
+        if t1 > t0:
+            prev = torch.cat([state[slot, :x.shape[1]].reshape(1, -1), xf[t0:t1 - 1]], dim=0)
+            cur = xf[t0:t1]
+            for m in range(mu.shape[0]):
+                out[m, t0:t1] = (cur + (prev - cur) * mu[m]).to(x.dtype)
+    return out
+
+
+def tail_update(state, x, channels, rows, cu, slots, num_seqs):
+    for t0, t1, slot in _seqs(cu, slots, num_seqs):
+        old = state[slot, :channels * rows].reshape(rows, channels).clone()
+        both = torch.cat([old, x[t0:t1, :channels].float()], dim=0)
+        state[slot, :channels * rows] = both[both.shape[0] - rows:].reshape(-1)
+
+
+def causal_conv(x, taps, state, seq_of_token, cu, slots, num_seqs, unit_channels=0, unit_group=0,
+                scaled_channels=0, scale=1.0, unit_eps=0.0, rest_group=256):
+    C, K = taps.shape
+    out = torch.empty((x.shape[0], C), dtype=torch.float32)
+    for t0, t1, slot in _seqs(cu, slots, num_seqs):
+        both = torch.cat([state[slot, :C * (K - 1)].reshape(K - 1, C), x[t0:t1, :C].float()], dim=0)
+        acc = torch.zeros(t1 - t0, C)
+        for j in range(K):
+            acc += both[j:j + t1 - t0] * taps[:, j]
+        out[t0:t1] = acc / (1.0 + torch.exp(-acc))
+    if unit_channels:
+        y = out[:, :unit_channels].reshape(x.shape[0], -1, unit_group)
+        y = y / torch.sqrt((y * y).sum(-1, keepdim=True) + unit_eps)
+        out[:, :unit_channels] = y.reshape(x.shape[0], unit_channels)
+        out[:, :scaled_channels] *= scale
+    return out
+
+
+def delta_scan(q, k, v, b_raw, a_raw, a_log, dt_bias, state, cu, slots, num_seqs, heads,
+               kv_heads, dk, dv):
+    T = q.shape[0]
+    out = torch.empty((T, heads * dv), dtype=torch.float32)
+    g = torch.exp(-torch.exp(a_log) * torch.nn.functional.softplus(a_raw + dt_bias))
+    beta = torch.sigmoid(b_raw)
+    for t0, t1, slot in _seqs(cu, slots, num_seqs):
+        S = state[slot, :heads * dv * dk].reshape(heads, dv, dk).clone()     # [head][value][key]
+        for t in range(t0, t1):
+            for h in range(heads):
+                j = h // (heads // kv_heads)
+                kt, qt = k[t, j * dk:(j + 1) * dk], q[t, j * dk:(j + 1) * dk]
+                S[h] = g[t, h] * S[h]
+                u = beta[t, h] * (v[t, h * dv:(h + 1) * dv] - S[h] @ kt)
+                S[h] = S[h] + torch.outer(u, kt)
+                out[t, h * dv:(h + 1) * dv] = S[h] @ qt
+        state[slot, :heads * dv * dk] = S.reshape(-1)
+    return out
+
+
+def decay_scan(r, k, v, z, w0, bonus, state, cu, slots, num_seqs, heads, d):
+    T = r.shape[0]
+    out = torch.empty((T, heads * d), dtype=torch.float32)
+    w = torch.exp(-torch.exp(z + w0)).reshape(T, heads, d)
+    u = bonus.reshape(heads, d)
+    rr, kk, vv = (t.reshape(T, heads, d) for t in (r, k, v))
+    for t0, t1, slot in _seqs(cu, slots, num_seqs):
+        S = state[slot, :heads * d * d].reshape(heads, d, d).clone()         # [head][value][key]
+        for t in range(t0, t1):
+            for h in range(heads):
+                vk = torch.outer(vv[t, h], kk[t, h])
+                out[t, h * d:(h + 1) * d] = (S[h] + vk * u[h]) @ rr[t, h]
+                S[h] = S[h] * w[t, h] + vk
+        state[slot, :heads * d * d] = S.reshape(-1)
+    return out
+
+
+def head_norm_gate(o, weight, gate, heads, dv, eps, out_dtype):
+    T = o.shape[0]
+    x = o.reshape(T, heads, dv)
+    x = x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
+    w = weight.reshape(heads, dv) if weight.numel() == heads * dv else weight.reshape(1, dv)
+    g = gate.float().reshape(T, heads, dv)
+    return (x * w * (g / (1.0 + torch.exp(-g)))).reshape(T, heads * dv).to(out_dtype)
 
 
 def linear(x, w, out_dtype=None, partials=False):
@@ -154,6 +259,8 @@ def install(monkeypatch) -> None:
     import rust_llm_inference_server_amd.engine.runner as runner
     for name in ("embed", "add_residual", "add_rmsnorm", "swiglu", "linear", "linear_swiglu",
                  "pending_linear", "can_fuse_norm_linear", "rope_kv_write", "rope_attention",
-                 "copy_pages", "attention_planner", "paged_attention", "sample_rows"):
+                 "copy_pages", "attention_planner", "paged_attention", "sample_rows",
+                 "clamped_glu", "weighted_sum", "soft_cap_", "shift_mix", "tail_update",
+                 "causal_conv", "delta_scan", "decay_scan", "head_norm_gate"):
         monkeypatch.setattr(ops, name, globals()[name])
     monkeypatch.setattr(runner, "default_device", lambda: torch.device("cpu"))

@@ -86,16 +86,24 @@ def time_mix(h: torch.Tensor, w: Dict[str, torch.Tensor], p: Dict[str, Any], eps
     gate = silu(mix("g") @ w["g"].T)
     decay = torch.exp(-torch.exp(torch.tanh(mix("w") @ w["w1"].T) @ w["w2"].T + w["w0"]))
     decay = decay.reshape(T, H, d)
-    u = w["u"].reshape(H, d)
-    S = torch.zeros(H, d, d, dtype=h.dtype)           # [head][key channel][value channel]
-    out = torch.zeros(T, H, d, dtype=h.dtype)
+    out = decayed_state(r, k, v, decay, w["u"].reshape(H, d))
+    out = rms(out, eps).reshape(T, H * d) * w["norm"] * gate
+    return out @ w["o"].T
+
+
+def decayed_state(r, k, v, decay, bonus, S=None):
+    """Per head a matrix S [key channel][value channel]: the token reads
+    ``(S + diag(bonus) k v^T)^T r``, then ``S <- diag(decay) S + k v^T``.
+    r, k, v, decay: (T, H, d); bonus (H, d).  ``S`` (H, d, d) is changed in place when given."""
+    T, H, d = r.shape
+    S = torch.zeros(H, d, d, dtype=r.dtype) if S is None else S
+    out = torch.zeros(T, H, d, dtype=r.dtype)
     for t in range(T):
         for head in range(H):
             kv = torch.outer(k[t, head], v[t, head])
-            out[t, head] = (S[head] + u[head].reshape(-1, 1) * kv).T @ r[t, head]
+            out[t, head] = (S[head] + bonus[head].reshape(-1, 1) * kv).T @ r[t, head]
             S[head] = decay[t, head].reshape(-1, 1) * S[head] + kv
-    out = rms(out, eps).reshape(T, H * d) * w["norm"] * gate
-    return out @ w["o"].T
+    return out
 
 
 def short_conv(x: torch.Tensor, taps: torch.Tensor) -> torch.Tensor:
@@ -124,8 +132,20 @@ def gated_delta(h: torch.Tensor, w: Dict[str, torch.Tensor], p: Dict[str, Any], 
     k = unit(k)
     beta = torch.sigmoid(h @ w["b"].T)                                     # (T, H)
     g = torch.exp(-torch.exp(w["A_log"]) * softplus(h @ w["a"].T + w["dt_bias"]))
-    S = torch.zeros(H, d, dv, dtype=h.dtype)
-    out = torch.zeros(T, H, dv, dtype=h.dtype)
+    out = delta_state(q, k, v, beta, g)
+    gate = silu(h @ w["g"].T).reshape(T, H, dv)
+    out = rms(out, eps) * w["norm"] * gate
+    return out.reshape(T, H * dv) @ w["o"].T
+
+
+def delta_state(q, k, v, beta, g, S=None):
+    """Per head a matrix S [key channel][value channel]: ``S <- g S``, then the token replaces
+    what its key reads, ``u = beta (v - S^T k)``, ``S <- S + k u^T``, and reads ``S^T q``.
+    q, k: (T, G, d); v: (T, H, dv); beta, g: (T, H); head h uses q/k head ``h // (H / G)``."""
+    T, G, d = q.shape
+    H, dv = v.shape[1], v.shape[2]
+    S = torch.zeros(H, d, dv, dtype=q.dtype) if S is None else S
+    out = torch.zeros(T, H, dv, dtype=q.dtype)
     for t in range(T):
         for head in range(H):
             j = head // (H // G)
@@ -133,9 +153,7 @@ def gated_delta(h: torch.Tensor, w: Dict[str, torch.Tensor], p: Dict[str, Any], 
             u = beta[t, head] * (v[t, head] - S[head].T @ k[t, j])
             S[head] = S[head] + torch.outer(k[t, j], u)
             out[t, head] = S[head].T @ q[t, j]
-    gate = silu(h @ w["g"].T).reshape(T, H, dv)
-    out = rms(out, eps) * w["norm"] * gate
-    return out.reshape(T, H * dv) @ w["o"].T
+    return out
 
 
 def clamped_glu(h: torch.Tensor, w: Dict[str, torch.Tensor], limit: float) -> torch.Tensor:
@@ -175,3 +193,16 @@ def forward(config: Dict[str, Any], weights: Dict[str, torch.Tensor], tokens: Li
     logits = offset_norm(x, weights["final.norm"], eps) @ weights["head"].T
     cap = config["logit_softcap"]
     return cap * torch.tanh(logits / cap)
+
+
+def greedy(config: Dict[str, Any], weights: Dict[str, torch.Tensor], prompt: List[int],
+           new_tokens: int):
+    """Greedy continuation, each token from a full forward pass; returns the tokens and, per
+    pick, the margin between the best and the second logit."""
+    tokens, margins = list(prompt), []
+    for _ in range(new_tokens):
+        last = forward(config, weights, tokens)[-1]
+        top = torch.topk(last, 2).values
+        margins.append(float(top[0] - top[1]))
+        tokens.append(int(torch.argmax(last)))
+    return tokens[len(prompt):], margins
