@@ -34,7 +34,16 @@ Weights are random (N(0, 0.02)), prompts are uniform random token ids.
     python bench.py --model llama-3.1-8b --batch 4 --context 32768 --prefill-tokens 8192 \
         --steps 32 --warmup 4 --skip-points
 
-run one of those workloads alone and print its own JSON line."""
+run one of those workloads alone and print its own JSON line.
+
+    python bench.py --designs [--sizes llama-3.2-1b,llama-3.2-3b] [--layers N]
+
+is another workload again: the Gipotar design (attention beside an RWKV-style time mix, gated
+delta rule, clamped gated unit; random weights) at the width, depth, feed-forward width,
+vocabulary and attention heads of a Llama preset, beside that preset itself: a prefill of
+``--prefill-tokens`` tokens in one step, and decode steps at batch 8 and 64 after 512-token
+prompts, each with the bytes a step has to read (weights once, the live requests' cache, and
+for Gipotar their state slots read and written) as a fraction of the HBM rate."""
 import argparse
 import copy
 import json
@@ -171,6 +180,144 @@ def run_requests(model, shape: Shape, reqs, new_tokens: int, budget: int, trials
     return best
 
 
+def gipotar_like(cfg: dict) -> dict:
+    """A Gipotar configuration at the sizes of a Llama preset: the same width, depth,
+    feed-forward width, vocabulary and attention heads; layers alternate between attention
+    beside a time mix (heads of 64) and the gated delta rule (heads of 128), each with a
+    feed-forward."""
+    W, d = cfg["hidden_size"], cfg["head_dim"]
+    mlp = {"kind": "dense", "ff": cfg["intermediate_size"], "limit": 7.0}
+    left = {"heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"], "dim": d,
+            "vdim": d, "rot": {"dims": d, "base": cfg["rope_theta"]}, "scale": d ** -0.5}
+    parallel = {"type": "parallel", "mlp": mlp,
+                "mixer": {"left": left, "left_scale": 0.7,
+                          "right": {"heads": W // 64, "dim": 64, "rank": 64}, "right_scale": 0.7}}
+    heads = max(1, W // 128)
+    delta = {"type": "delta", "mlp": mlp,
+             "mixer": {"heads": heads, "kv_heads": max(1, heads // 2), "dim": 128, "vdim": 128,
+                       "conv": 4}}
+    return {"architecture": "Gipotar", "vocab": cfg["vocab_size"], "width": W,
+            "embedding": {"scale": 1.0}, "residual_mult": 1.0, "norm": {"eps": 1e-5},
+            "logit_softcap": 30.0,
+            "layers": [copy.deepcopy(parallel if i % 2 == 0 else delta)
+                       for i in range(cfg["num_hidden_layers"])]}
+
+
+def step_bytes_of(model, batch: int, mean_context: float) -> float:
+    """What a decode step of any model has to move: every tensor its parts hold once (the
+    embedding table only where the head shares it), each live request's cached positions, and
+    its state slot read and written."""
+    seen, total = set(), 0
+    for t in model._tensors():
+        if t.data_ptr() not in seen:
+            seen.add(t.data_ptr())
+            total += t.numel() * t.element_size()
+    table = model.embedding.weight
+    if model.head.weight.data_ptr() != table.data_ptr():
+        total -= table.numel() * table.element_size()
+    per_position = sum(len(g.writer_runs) * g.request.bytes_per_token(model.act_dtype)
+                       for g in model.cache_groups)
+    return total + batch * (mean_context * per_position + 2 * model.state_bytes)
+
+
+def time_prefill(model, prompt, runs: int = 8) -> float:
+    """Seconds of one prompt in one step (the best of ``runs``, of which the later ones replay
+    the captured step)."""
+    import torch
+    from rust_llm_inference_server_amd.engine import ModelRunner, StepEntry
+    T = len(prompt)
+    runner = ModelRunner(model, num_pages=-(-T // PAGE) + 1, page_size=PAGE, max_num_seqs=1)
+    times = []
+    for _ in range(runs):
+        runner.reserve(0, T)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        runner.step([StepEntry(0, prompt, [T - 1])])
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+        runner.free(0)
+    return min(times[1:] or times)
+
+
+def time_decode(model, prompts_of_batch, steps: int, warmup: int):
+    """(tokens/s, ms/step, mean context) of ``steps`` decode steps of the requests
+    ``prompts_of_batch``, all prompts prefilled in one step, the decode steps captured
+    beforehand."""
+    import torch
+    from rust_llm_inference_server_amd.config import EngineConfig
+    from rust_llm_inference_server_amd.engine import Engine
+    from rust_llm_inference_server_amd.sampling import SamplingParams
+    batch, prompt_len = len(prompts_of_batch), len(prompts_of_batch[0])
+    new_tokens = steps + warmup + 3
+    context = prompt_len + new_tokens
+    engine = Engine(model, EngineConfig(
+        max_num_seqs=batch, max_batched_tokens=batch * prompt_len,
+        num_pages=batch * (-(-context // PAGE) + 1) + 8, block_size=PAGE, max_seq_len=context + 8,
+        watermark_pages=0))
+    sp = SamplingParams(max_tokens=new_tokens, ignore_eos=True)
+    engine.runner.capture_decode_steps(longest=context + 8, max_batch=batch)
+    for p in prompts_of_batch:
+        engine.add_request(p, sp)
+    while engine.stats().prefill_tokens < batch * prompt_len or engine.stats().waiting:
+        engine.step()
+    for _ in range(warmup):
+        engine.step()
+    torch.cuda.synchronize()
+    before = copy.copy(engine.stats())
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        engine.step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    after = engine.stats()
+    if after.generated_tokens - before.generated_tokens != batch * steps:
+        raise RuntimeError("the timed steps were not pure decode steps of the whole batch")
+    mean_ctx = prompt_len + (before.generated_tokens + after.generated_tokens) / 2 / batch
+    return batch * steps / dt, dt / steps * 1e3, mean_ctx
+
+
+def compare_designs(args) -> int:
+    """The Gipotar design beside the Llama preset of the same sizes: one JSON line."""
+    import torch
+    from rust_llm_inference_server_amd.config import preset_dict
+    from rust_llm_inference_server_amd.engine import random_model
+    g = torch.Generator().manual_seed(0)
+    T, new, warm = args.prefill_tokens, min(args.steps, 64), min(args.warmup, 8)
+    results = {}
+    for size in args.sizes.split(","):
+        base = preset_dict(size)
+        if args.layers:
+            base["num_hidden_layers"] = args.layers
+        longest = max(T, args.points_context + new + warm + 16) + 64
+        base["max_position_embeddings"] = min(base["max_position_embeddings"], longest)
+        for design, cfg in (("llama", base), ("gipotar", gipotar_like(base))):
+            vocab = base["vocab_size"]
+            model = random_model(cfg, seed=0, dtype=args.dtype, max_positions=longest)
+            torch.cuda.synchronize()
+            r = {"layers": base["num_hidden_layers"]}
+            s = time_prefill(model, torch.randint(0, vocab, (T,), generator=g).tolist())
+            r["prefill_tok_s"], r["prefill_ms"] = round(T / s, 1), round(s * 1e3, 3)
+            for b in (8, 64):
+                reqs = [torch.randint(0, vocab, (args.points_context,), generator=g).tolist()
+                        for _ in range(b)]
+                v, ms, ctx = time_decode(model, reqs, new, warm)
+                frac = step_bytes_of(model, b, ctx) / (ms * 1e-3) / 1e9 / HBM_GBPS
+                r[f"decode_b{b}_tok_s"], r[f"decode_b{b}_ms"] = round(v, 1), round(ms, 4)
+                r[f"decode_b{b}_hbm_frac"] = round(frac, 4)
+            results[f"{size}/{design}"] = r
+            say(f"{size} {design}: {r}")
+            del model
+            torch.cuda.empty_cache()
+    print(json.dumps({
+        "metric": "prefill and decode tok/s, Gipotar beside Llama at equal sizes",
+        "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic (random weights N(0,0.02), uniform random token ids)",
+        "config": {"sizes": args.sizes, "prefill_tokens": T, "decode_prompt": args.points_context,
+                   "decode_steps": new, "page_size": PAGE},
+        "results": results}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -200,6 +347,10 @@ def main() -> int:
     ap.add_argument("--min-prompt", type=int, default=128)
     ap.add_argument("--max-prompt", type=int, default=2048)
     ap.add_argument("--new-tokens", type=int, default=256)
+    ap.add_argument("--designs", action="store_true",
+                    help="time the Gipotar design beside the Llama presets of --sizes instead")
+    ap.add_argument("--sizes", default="llama-3.2-1b,llama-3.2-3b",
+                    help="presets whose sizes the two designs of --designs are built at")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (single-GPU engine)")
@@ -224,6 +375,9 @@ def main() -> int:
     def random_requests(n, lo, hi, vocab):
         lens = torch.randint(lo, hi + 1, (n,), generator=g).tolist()
         return [torch.randint(0, vocab, (m,), generator=g).tolist() for m in lens]
+
+    if args.designs:
+        return compare_designs(args)
 
     if args.serve:
         # ---- one workload of requests through the engine, alone ------------------------------

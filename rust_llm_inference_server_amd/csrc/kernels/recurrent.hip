@@ -9,10 +9,11 @@
 // step before left, whatever else is in the batch; a sequence at position 0 finds zeros (the
 // runner clears the slot), which are the zeros in front of a sequence's first token.
 //
-// The matrix state is walked by one wave per (sequence, head, value channel j): lane i holds
-// S[i][j] (and i + 64, ... for more than 64 key channels), a token's read-out is one sum over
-// the wave, and nothing is shared between waves, so the columns of a head spread over the chip.
-// State layout per head: [value channel][key channel], so a wave's column is contiguous.
+// The matrix state is walked by one wave per (sequence, head, four value channels): lane i
+// holds S[i][j] of each (and i + 64, ... for more than 64 key channels), a token's read-out is
+// a sum over the wave, and nothing is shared between waves, so the columns of a head spread
+// over the chip.  State layout per head: [value channel][key channel], so a wave's columns are
+// contiguous.
 #include "common.h"
 
 namespace {
@@ -132,11 +133,56 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(
   }
 }
 
-// ------------------------------------------------------------- gated delta rule
-// Per token and head, with one decay g and one step size beta per head:
+// ------------------------------------------------------------------ the two scans
+// Sum over the 64 lanes of a wave, every lane gets it: four data-parallel-primitive adds inside
+// rows of 16 lanes (neighbour, pair, the other quad, the other half-row) and the two half
+// swaps; no trip through LDS.  The order of the additions is fixed.
+template <int CTRL>
+__device__ __forceinline__ float dpp_from(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float lanes_sum(float v) {
+  v += dpp_from<0xB1>(v);    // quad_perm [1, 0, 3, 2]
+  v += dpp_from<0x4E>(v);    // quad_perm [2, 3, 0, 1]
+  v += dpp_from<0x141>(v);   // row_half_mirror
+  v += dpp_from<0x140>(v);   // row_mirror
+  v = xor16_sum(v);
+  return xor32_sum(v);
+}
+
+// Four sums over the wave at once, for values a wave holds per lane for four columns: lanes
+// trade columns with their neighbour and their neighbour's neighbour, so that lane l carries on
+// with column l % 4 alone, and the steps that follow (4 and 8 lanes round the row, the half
+// swaps) keep that class.  Lane l ends with the whole sum of column l % 4: ten adds and moves
+// for four sums where four separate sums take twenty-four.  The order of the additions is fixed.
+__device__ __forceinline__ float lanes_sum4(const float (&p)[4], int lane) {
+  const bool odd = lane & 1, high = lane & 2;
+  float a01 = odd ? p[1] : p[0];
+  a01 += dpp_from<0xB1>(odd ? p[0] : p[1]);
+  float a23 = odd ? p[3] : p[2];
+  a23 += dpp_from<0xB1>(odd ? p[2] : p[3]);
+  float a = high ? a23 : a01;
+  a += dpp_from<0x4E>(high ? a01 : a23);
+  a += dpp_from<0x124>(a);   // row_ror 4
+  a += dpp_from<0x128>(a);   // row_ror 8
+  a = xor16_sum(a);
+  return xor32_sum(a);
+}
+
+// A wave walks kCols value channels of one (sequence, head): lane i holds S[i][j] of each (and
+// i + 64, ... for more than 64 key channels), so what a token brings per key channel is loaded
+// once for all of them and their sums over the wave interleave.  What does not depend on the
+// state (decays, step sizes, the products of a token's own vectors) is made one token ahead,
+// while the token before it waits for its sums.  No load stands under a condition: lanes and
+// columns past the end read a clamped address and their values are zeroed or not stored.
+constexpr int kCols = 4;
+
+// Gated delta rule.  Per token and head, with one decay g and one step size beta per head:
 //   S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q.
 // g = exp(-exp(A_log) * softplus(a + dt_bias)), beta = sigmoid(b), from the raw projections.
-// Each column j of S is independent: u_j = beta (v_j - sum_i S_ij k_i), and so on.
+// Column j of S is independent of the others.  With d1 = S^T k and d2 = S^T q of the state
+// before the token, u_j = beta (v_j - g d1_j) and o_j = g d2_j + (k . q) u_j, so both sums
+// are over the old state and wait for nothing but each other.
 template <int KR>
 __global__ __launch_bounds__(256) void delta_scan_kernel(
     float* __restrict__ out, long long ldo, const float* __restrict__ q, const float* __restrict__ k,
@@ -147,76 +193,100 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
     int dv) {
   const int lane = threadIdx.x % kWave;
   const int wave = threadIdx.x / kWave;
-  const int cols_per_block = blockDim.x / kWave;
-  const int j = blockIdx.x * cols_per_block + wave;
+  const int j0 = (blockIdx.x * (blockDim.x / kWave) + wave) * kCols;
   const int head = blockIdx.y;
   const int s = blockIdx.z;
-  if (j >= dv) return;
+  if (j0 >= dv) return;
   const int kh = head / (heads / kv_heads);
   const int t0 = cu[s], t1 = cu[s + 1];
-  float* col = state + (long long)slots[s] * state_stride + ((long long)head * dv + j) * dk;
-  float S[KR];
+  float* base = state + (long long)slots[s] * state_stride + (long long)head * dv * dk;
+  int idx[KR];
+  float live[KR];
 #pragma unroll
   for (int r = 0; r < KR; ++r) {
     const int i = lane + r * kWave;
-    S[r] = i < dk ? col[i] : 0.f;
+    idx[r] = i < dk ? i : dk - 1;
+    live[r] = i < dk ? 1.f : 0.f;
   }
+  int col[kCols];
+#pragma unroll
+  for (int c = 0; c < kCols; ++c) col[c] = j0 + c < dv ? j0 + c : dv - 1;
+  float S[kCols][KR];
+#pragma unroll
+  for (int c = 0; c < kCols; ++c)
+#pragma unroll
+    for (int r = 0; r < KR; ++r) S[c][r] = base[(long long)col[c] * dk + idx[r]] * live[r];
   const float neg_a = -expf(a_log[head]);
   const float bias = dt_bias[head];
-  float kn[KR], qn[KR], vn = 0.f, bn = 0.f, an = 0.f;
+  // the token ahead: its vectors, and what follows from them alone
+  float kn[KR], qn[KR], vn[kCols], gn = 0.f, betan = 0.f, kqn = 0.f;
   auto fetch = [&](int t) {
     const float* kt = k + (long long)t * ldqkv + kh * dk;
     const float* qt = q + (long long)t * ldqkv + kh * dk;
+    float kq = 0.f;
 #pragma unroll
     for (int r = 0; r < KR; ++r) {
-      const int i = lane + r * kWave;
-      kn[r] = i < dk ? kt[i] : 0.f;
-      qn[r] = i < dk ? qt[i] : 0.f;
+      kn[r] = kt[idx[r]] * live[r];
+      qn[r] = qt[idx[r]] * live[r];
+      kq += kn[r] * qn[r];
     }
-    vn = v[(long long)t * ldqkv + head * dv + j];
-    bn = b_raw[(long long)t * ldba + head];
-    an = a_raw[(long long)t * ldba + head];
+#pragma unroll
+    for (int c = 0; c < kCols; ++c) vn[c] = v[(long long)t * ldqkv + head * dv + col[c]];
+    betan = sigmoidf_(b_raw[(long long)t * ldba + head]);
+    gn = expf(neg_a * softplusf_(a_raw[(long long)t * ldba + head] + bias));
+    kqn = lanes_sum(kq);
   };
   if (t0 < t1) fetch(t0);
   for (int t = t0; t < t1; ++t) {
-    float kc[KR], qc[KR];
+    float kc[KR], qc[KR], vc[kCols];
 #pragma unroll
     for (int r = 0; r < KR; ++r) {
       kc[r] = kn[r];
       qc[r] = qn[r];
     }
-    const float vc = vn, bc = bn, ac = an;
-    if (t + 1 < t1) fetch(t + 1);
-    const float g = expf(neg_a * softplusf_(ac + bias));
-    const float beta = sigmoidf_(bc);
-    float dot = 0.f;
 #pragma unroll
-    for (int r = 0; r < KR; ++r) {
-      S[r] *= g;
-      dot += S[r] * kc[r];
-    }
-    dot = wave_sum(dot);
-    const float u = beta * (vc - dot);
-    float o = 0.f;
+    for (int c = 0; c < kCols; ++c) vc[c] = vn[c];
+    const float g = gn, beta = betan, kq = kqn;
+    fetch(t + 1 < t1 ? t + 1 : t);
+    float d1[kCols], d2[kCols];
 #pragma unroll
-    for (int r = 0; r < KR; ++r) {
-      S[r] += kc[r] * u;
-      o += S[r] * qc[r];
+    for (int c = 0; c < kCols; ++c) {
+      d1[c] = 0.f;
+      d2[c] = 0.f;
+#pragma unroll
+      for (int r = 0; r < KR; ++r) {
+        d1[c] += S[c][r] * kc[r];
+        d2[c] += S[c][r] * qc[r];
+      }
     }
-    o = wave_sum(o);
-    if (lane == 0) out[(long long)t * ldo + head * dv + j] = o;
+#pragma unroll
+    for (int c = 0; c < kCols; ++c) {
+      d1[c] = lanes_sum(d1[c]);
+      d2[c] = lanes_sum(d2[c]);
+    }
+#pragma unroll
+    for (int c = 0; c < kCols; ++c) {
+      const float u = beta * (vc[c] - g * d1[c]);
+#pragma unroll
+      for (int r = 0; r < KR; ++r) S[c][r] = g * S[c][r] + kc[r] * u;
+      if (lane == c && j0 + c < dv)
+        out[(long long)t * ldo + head * dv + j0 + c] = g * d2[c] + kq * u;
+    }
   }
 #pragma unroll
-  for (int r = 0; r < KR; ++r) {
-    const int i = lane + r * kWave;
-    if (i < dk) col[i] = S[r];
-  }
+  for (int c = 0; c < kCols; ++c)
+    if (j0 + c < dv) {
+#pragma unroll
+      for (int r = 0; r < KR; ++r)
+        if (lane + r * kWave < dk) base[(long long)(j0 + c) * dk + lane + r * kWave] = S[c][r];
+    }
 }
 
-// ------------------------------------------------- decayed state with a bonus for the present
-// Per token and head, with a decay per key channel w_i = exp(-exp(z_i + w0_i)):
+// Decayed state with a bonus for the present.  Per token and head, with a decay per key channel
+// w_i = exp(-exp(z_i + w0_i)):
 //   o = (S + diag(u) k v^T)^T r;  S <- diag(w) S + k v^T.
 // Keys, values and receptances have one size `d` here; z is the raw low-rank projection.
+// o_j = sum_i r_i S_ij + (sum_i r_i u_i k_i) v_j: the second sum does not depend on the state.
 template <int KR>
 __global__ __launch_bounds__(256) void decay_scan_kernel(
     float* __restrict__ out, const float* __restrict__ r_in, const float* __restrict__ k_in,
@@ -226,60 +296,343 @@ __global__ __launch_bounds__(256) void decay_scan_kernel(
     int d) {
   const int lane = threadIdx.x % kWave;
   const int wave = threadIdx.x / kWave;
-  const int cols_per_block = blockDim.x / kWave;
-  const int j = blockIdx.x * cols_per_block + wave;
+  const int j0 = (blockIdx.x * (blockDim.x / kWave) + wave) * kCols;
   const int head = blockIdx.y;
   const int s = blockIdx.z;
-  if (j >= d) return;
+  if (j0 >= d) return;
   const int t0 = cu[s], t1 = cu[s + 1];
-  float* col = state + (long long)slots[s] * state_stride + ((long long)head * d + j) * d;
-  float S[KR], u[KR], base[KR];
+  float* base = state + (long long)slots[s] * state_stride + (long long)head * d * d;
+  int idx[KR];
+  float live[KR];
 #pragma unroll
   for (int r = 0; r < KR; ++r) {
     const int i = lane + r * kWave;
-    S[r] = i < d ? col[i] : 0.f;
-    u[r] = i < d ? bonus[head * d + i] : 0.f;
-    base[r] = i < d ? w0[head * d + i] : 0.f;
+    idx[r] = i < d ? i : d - 1;
+    live[r] = i < d ? 1.f : 0.f;
   }
-  float rn[KR], kn[KR], zn[KR], vn = 0.f;
+  int col[kCols];
+#pragma unroll
+  for (int c = 0; c < kCols; ++c) col[c] = j0 + c < d ? j0 + c : d - 1;
+  float S[kCols][KR], u[KR], w_base[KR];
+#pragma unroll
+  for (int r = 0; r < KR; ++r) {
+    u[r] = bonus[head * d + idx[r]];
+    w_base[r] = w0[head * d + idx[r]];
+#pragma unroll
+    for (int c = 0; c < kCols; ++c) S[c][r] = base[(long long)col[c] * d + idx[r]] * live[r];
+  }
+  float rn[KR], kn[KR], wn[KR], vn[kCols], rukn = 0.f;
   auto fetch = [&](int t) {
     const long long row = (long long)t * ld + head * d;
+    float ruk = 0.f;
 #pragma unroll
     for (int r = 0; r < KR; ++r) {
-      const int i = lane + r * kWave;
-      rn[r] = i < d ? r_in[row + i] : 0.f;
-      kn[r] = i < d ? k_in[row + i] : 0.f;
-      zn[r] = i < d ? z_in[row + i] : 0.f;
+      rn[r] = r_in[row + idx[r]] * live[r];
+      kn[r] = k_in[row + idx[r]] * live[r];
+      wn[r] = expf(-expf(z_in[row + idx[r]] + w_base[r]));
+      ruk += rn[r] * u[r] * kn[r];
     }
-    vn = v_in[row + j];
+#pragma unroll
+    for (int c = 0; c < kCols; ++c) vn[c] = v_in[row + col[c]];
+    rukn = lanes_sum(ruk);
   };
   if (t0 < t1) fetch(t0);
   for (int t = t0; t < t1; ++t) {
-    float rc[KR], kc[KR], zc[KR];
+    float rc[KR], kc[KR], wc[KR], vc[kCols];
 #pragma unroll
     for (int r = 0; r < KR; ++r) {
       rc[r] = rn[r];
       kc[r] = kn[r];
-      zc[r] = zn[r];
+      wc[r] = wn[r];
     }
-    const float vc = vn;
-    if (t + 1 < t1) fetch(t + 1);
-    float o = 0.f;
 #pragma unroll
-    for (int r = 0; r < KR; ++r) {
-      const float kv = kc[r] * vc;
-      const float w = expf(-expf(zc[r] + base[r]));
-      o += rc[r] * (S[r] + u[r] * kv);
-      S[r] = w * S[r] + kv;
+    for (int c = 0; c < kCols; ++c) vc[c] = vn[c];
+    const float ruk = rukn;
+    fetch(t + 1 < t1 ? t + 1 : t);
+    float o[kCols];
+#pragma unroll
+    for (int c = 0; c < kCols; ++c) {
+      o[c] = 0.f;
+#pragma unroll
+      for (int r = 0; r < KR; ++r) {
+        o[c] += rc[r] * S[c][r];
+        S[c][r] = wc[r] * S[c][r] + kc[r] * vc[c];
+      }
     }
-    o = wave_sum(o);
-    if (lane == 0) out[(long long)t * ld + head * d + j] = o;
+#pragma unroll
+    for (int c = 0; c < kCols; ++c) o[c] = lanes_sum(o[c]);
+#pragma unroll
+    for (int c = 0; c < kCols; ++c)
+      if (lane == c && j0 + c < d) out[(long long)t * ld + head * d + j0 + c] = o[c] + ruk * vc[c];
   }
+#pragma unroll
+  for (int c = 0; c < kCols; ++c)
+    if (j0 + c < d) {
+#pragma unroll
+      for (int r = 0; r < KR; ++r)
+        if (lane + r * kWave < d) base[(long long)(j0 + c) * d + lane + r * kWave] = S[c][r];
+    }
+}
+
+// ------------------------------------------------------- the scans over long runs of tokens
+// The kernels above ask for a token's vectors one token ahead, which hides the arithmetic of one
+// token and no more: over a prompt's portion every token would wait out a trip to memory.  The
+// forms below are for steps in which some sequence brings many tokens.  A workgroup (four waves,
+// sixteen value channels of one head) asks for a whole tile of tokens at once, keeps it in
+// registers while its waves walk the tile before from LDS, each over its own columns, and then
+// moves it to LDS with everything that follows from a token alone made on the way (decays and
+// step sizes; columns and tokens past the end read clamped addresses).  A token's four sums over
+// the wave are formed together (lanes_sum4), so a row comes out as above to rounding, not to
+// the bit.
+template <int KR>
+struct ScanTile {
+  static constexpr int kTokens = KR == 4 ? 16 : 32;
+  static constexpr int kKeys = KR * kWave;
+};
+
+template <int KR>
+__global__ __launch_bounds__(256) void delta_scan_tiled_kernel(
+    float* __restrict__ out, long long ldo, const float* __restrict__ q, const float* __restrict__ k,
+    const float* __restrict__ v, long long ldqkv, const float* __restrict__ b_raw,
+    const float* __restrict__ a_raw, long long ldba, const float* __restrict__ a_log,
+    const float* __restrict__ dt_bias, float* __restrict__ state, long long state_stride,
+    const int* __restrict__ cu, const int* __restrict__ slots, int heads, int kv_heads, int dk,
+    int dv) {
+  constexpr int TT = ScanTile<KR>::kTokens, DK = ScanTile<KR>::kKeys, CB = 4 * kCols;
+  __shared__ float tk[TT][DK], tq[TT][DK], tv[TT][CB], tg[TT], tb[TT];
+  const int lane = threadIdx.x % kWave;
+  const int wave = threadIdx.x / kWave;
+  const int jb = blockIdx.x * CB;                 // the workgroup's first column
+  const int j0 = jb + wave * kCols;
+  const int head = blockIdx.y;
+  const int s = blockIdx.z;
+  const int kh = head / (heads / kv_heads);
+  const int t0 = cu[s], t1 = cu[s + 1];
+  float* base = state + (long long)slots[s] * state_stride + (long long)head * dv * dk;
+  int idx[KR];
+  float live[KR];
 #pragma unroll
   for (int r = 0; r < KR; ++r) {
     const int i = lane + r * kWave;
-    if (i < d) col[i] = S[r];
+    idx[r] = i < dk ? i : dk - 1;
+    live[r] = i < dk ? 1.f : 0.f;
   }
+  float S[kCols][KR];
+#pragma unroll
+  for (int c = 0; c < kCols; ++c) {
+    const int col = j0 + c < dv ? j0 + c : dv - 1;
+#pragma unroll
+    for (int r = 0; r < KR; ++r) S[c][r] = base[(long long)col * dk + idx[r]] * live[r];
+  }
+  const float neg_a = -expf(a_log[head]);
+  const float bias = dt_bias[head];
+  // A tile's values wait in registers while the tile before is walked: every load of a tile is
+  // asked for at once, and none of them is waited for before the walk in front of it is over.
+  constexpr int PER = TT * DK / 256, PERV = TT * CB / 256;
+  static_assert(TT * DK % 256 == 0 && TT * CB % 256 == 0 && TT <= 256, "tile sizes");
+  float rk[PER], rq[PER], rv[PERV], rb = 0.f, rg = 0.f;
+  auto ask = [&](int tile) {
+    const int n = min(TT, t1 - tile);
+#pragma unroll
+    for (int p = 0; p < PER; ++p) {
+      const int e = threadIdx.x + p * 256, tt = e / DK, i = e % DK;
+      const long long row = (long long)(tile + (tt < n ? tt : n - 1)) * ldqkv + kh * dk;
+      const int ic = i < dk ? i : dk - 1;
+      const float keep = (tt < n && i < dk) ? 1.f : 0.f;
+      rk[p] = k[row + ic] * keep;
+      rq[p] = q[row + ic] * keep;
+    }
+#pragma unroll
+    for (int p = 0; p < PERV; ++p) {
+      const int e = threadIdx.x + p * 256, tt = e / CB, c = e % CB;
+      const int col = jb + c < dv ? jb + c : dv - 1;
+      rv[p] = v[(long long)(tile + (tt < n ? tt : n - 1)) * ldqkv + head * dv + col];
+    }
+    const int tt = threadIdx.x < TT ? threadIdx.x : TT - 1;
+    const long long row = (long long)(tile + (tt < n ? tt : n - 1)) * ldba + head;
+    rb = b_raw[row];
+    rg = a_raw[row];
+  };
+  if (t0 < t1) ask(t0);
+  for (int tile = t0; tile < t1; tile += TT) {
+    const int n = min(TT, t1 - tile);
+    __syncthreads();                               // the tile before has been walked
+#pragma unroll
+    for (int p = 0; p < PER; ++p) {
+      const int e = threadIdx.x + p * 256;
+      tk[e / DK][e % DK] = rk[p];
+      tq[e / DK][e % DK] = rq[p];
+    }
+#pragma unroll
+    for (int p = 0; p < PERV; ++p) {
+      const int e = threadIdx.x + p * 256;
+      tv[e / CB][e % CB] = rv[p];
+    }
+    if (threadIdx.x < TT) {
+      tb[threadIdx.x] = sigmoidf_(rb);
+      tg[threadIdx.x] = expf(neg_a * softplusf_(rg + bias));
+    }
+    __syncthreads();
+    ask(tile + TT < t1 ? tile + TT : tile);
+    // Lane l gathers the read-out of token (l / 4) of a group of sixteen for column l % 4 and
+    // stores it when the group is through: one store a group, not four a token.
+    float gathered = 0.f;
+    for (int tt = 0; tt < n; ++tt) {
+      float kc[KR], qc[KR], kq = 0.f;
+#pragma unroll
+      for (int r = 0; r < KR; ++r) {
+        kc[r] = tk[tt][lane + r * kWave];
+        qc[r] = tq[tt][lane + r * kWave];
+        kq += kc[r] * qc[r];
+      }
+      const float g = tg[tt], beta = tb[tt];
+      const float v_own = tv[tt][wave * kCols + (lane & 3)];
+      float d1[kCols], d2[kCols];
+#pragma unroll
+      for (int c = 0; c < kCols; ++c) {
+        d1[c] = 0.f;
+        d2[c] = 0.f;
+#pragma unroll
+        for (int r = 0; r < KR; ++r) {
+          d1[c] += S[c][r] * kc[r];
+          d2[c] += S[c][r] * qc[r];
+        }
+      }
+      kq = lanes_sum(kq);
+      const float s1 = lanes_sum4(d1, lane), s2 = lanes_sum4(d2, lane);
+      const float u_own = beta * (v_own - g * s1);          // of column lane % 4
+      if ((lane >> 2) == (tt & 15)) gathered = g * s2 + kq * u_own;
+      const float u[kCols] = {dpp_from<0x00>(u_own), dpp_from<0x55>(u_own), dpp_from<0xAA>(u_own),
+                              dpp_from<0xFF>(u_own)};       // each column's, to every lane
+#pragma unroll
+      for (int c = 0; c < kCols; ++c)
+#pragma unroll
+        for (int r = 0; r < KR; ++r) S[c][r] = g * S[c][r] + kc[r] * u[c];
+      if ((tt & 15) == 15 || tt == n - 1) {
+        const int token = (tt & ~15) + (lane >> 2);
+        if (token <= tt && j0 + (lane & 3) < dv)
+          out[(long long)(tile + token) * ldo + head * dv + j0 + (lane & 3)] = gathered;
+      }
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < kCols; ++c)
+    if (j0 + c < dv) {
+#pragma unroll
+      for (int r = 0; r < KR; ++r)
+        if (lane + r * kWave < dk) base[(long long)(j0 + c) * dk + lane + r * kWave] = S[c][r];
+    }
+}
+
+template <int KR>
+__global__ __launch_bounds__(256) void decay_scan_tiled_kernel(
+    float* __restrict__ out, const float* __restrict__ r_in, const float* __restrict__ k_in,
+    const float* __restrict__ v_in, const float* __restrict__ z_in, long long ld,
+    const float* __restrict__ w0, const float* __restrict__ bonus, float* __restrict__ state,
+    long long state_stride, const int* __restrict__ cu, const int* __restrict__ slots, int heads,
+    int d) {
+  constexpr int TT = ScanTile<KR>::kTokens / 2, DK = ScanTile<KR>::kKeys, CB = 4 * kCols;
+  __shared__ float tr[TT][DK], tk[TT][DK], tw[TT][DK], tv[TT][CB];
+  const int lane = threadIdx.x % kWave;
+  const int wave = threadIdx.x / kWave;
+  const int jb = blockIdx.x * CB;
+  const int j0 = jb + wave * kCols;
+  const int head = blockIdx.y;
+  const int s = blockIdx.z;
+  const int t0 = cu[s], t1 = cu[s + 1];
+  float* base = state + (long long)slots[s] * state_stride + (long long)head * d * d;
+  float S[kCols][KR], u[KR];
+#pragma unroll
+  for (int r = 0; r < KR; ++r) {
+    const int i = lane + r * kWave;
+    const int ic = i < d ? i : d - 1;
+    const float keep = i < d ? 1.f : 0.f;
+    u[r] = bonus[head * d + ic];
+#pragma unroll
+    for (int c = 0; c < kCols; ++c) {
+      const int col = j0 + c < d ? j0 + c : d - 1;
+      S[c][r] = base[(long long)col * d + ic] * keep;
+    }
+  }
+  constexpr int PER = TT * DK / 256, PERV = (TT * CB + 255) / 256;
+  static_assert(TT * DK % 256 == 0, "tile sizes");
+  float rr[PER], rk[PER], rz[PER], rv[PERV];
+  auto ask = [&](int tile) {
+    const int n = min(TT, t1 - tile);
+#pragma unroll
+    for (int p = 0; p < PER; ++p) {
+      const int e = threadIdx.x + p * 256, tt = e / DK, i = e % DK;
+      const long long row = (long long)(tile + (tt < n ? tt : n - 1)) * ld + head * d;
+      const int ic = i < d ? i : d - 1;
+      const float keep = (tt < n && i < d) ? 1.f : 0.f;
+      rr[p] = r_in[row + ic] * keep;
+      rk[p] = k_in[row + ic] * keep;
+      rz[p] = z_in[row + ic] + w0[head * d + ic];
+    }
+#pragma unroll
+    for (int p = 0; p < PERV; ++p) {
+      const int e = min(threadIdx.x + p * 256, TT * CB - 1), tt = e / CB, c = e % CB;
+      const int col = jb + c < d ? jb + c : d - 1;
+      rv[p] = v_in[(long long)(tile + (tt < n ? tt : n - 1)) * ld + head * d + col];
+    }
+  };
+  if (t0 < t1) ask(t0);
+  for (int tile = t0; tile < t1; tile += TT) {
+    const int n = min(TT, t1 - tile);
+    __syncthreads();                               // the tile before has been walked
+#pragma unroll
+    for (int p = 0; p < PER; ++p) {
+      const int e = threadIdx.x + p * 256;
+      tr[e / DK][e % DK] = rr[p];
+      tk[e / DK][e % DK] = rk[p];
+      tw[e / DK][e % DK] = expf(-expf(rz[p]));
+    }
+#pragma unroll
+    for (int p = 0; p < PERV; ++p) {
+      const int e = threadIdx.x + p * 256;
+      if (e < TT * CB) tv[e / CB][e % CB] = rv[p];
+    }
+    __syncthreads();
+    ask(tile + TT < t1 ? tile + TT : tile);
+    float gathered = 0.f;                          // as in the kernel above
+    for (int tt = 0; tt < n; ++tt) {
+      float rc[KR], kc[KR], wc[KR], ruk = 0.f;
+#pragma unroll
+      for (int r = 0; r < KR; ++r) {
+        rc[r] = tr[tt][lane + r * kWave];
+        kc[r] = tk[tt][lane + r * kWave];
+        wc[r] = tw[tt][lane + r * kWave];
+        ruk += rc[r] * u[r] * kc[r];
+      }
+      const float v_own = tv[tt][wave * kCols + (lane & 3)];
+      float o[kCols];
+#pragma unroll
+      for (int c = 0; c < kCols; ++c) {
+        const float vc = tv[tt][wave * kCols + c];
+        o[c] = 0.f;
+#pragma unroll
+        for (int r = 0; r < KR; ++r) {
+          o[c] += rc[r] * S[c][r];
+          S[c][r] = wc[r] * S[c][r] + kc[r] * vc;
+        }
+      }
+      ruk = lanes_sum(ruk);
+      const float total = lanes_sum4(o, lane);
+      if ((lane >> 2) == (tt & 15)) gathered = total + ruk * v_own;
+      if ((tt & 15) == 15 || tt == n - 1) {
+        const int token = (tt & ~15) + (lane >> 2);
+        if (token <= tt && j0 + (lane & 3) < d)
+          out[(long long)(tile + token) * ld + head * d + j0 + (lane & 3)] = gathered;
+      }
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < kCols; ++c)
+    if (j0 + c < d) {
+#pragma unroll
+      for (int r = 0; r < KR; ++r)
+        if (lane + r * kWave < d) base[(long long)(j0 + c) * d + lane + r * kWave] = S[c][r];
+    }
 }
 
 // --------------------------------------------------- per-head RMS norm, weight and gate
@@ -377,22 +730,33 @@ RLIS_API int rlis_delta_scan(float* out, long long ldo, const float* q, const fl
                              const float* a_raw, long long ldba, const float* a_log,
                              const float* dt_bias, float* state, long long state_stride,
                              const int* cu, const int* slots, int num_seqs, int heads,
-                             int kv_heads, int dk, int dv, hipStream_t stream) {
+                             int kv_heads, int dk, int dv, int tiled, hipStream_t stream) {
   RLIS_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dk > 0 && dv > 0,
                "delta_scan: bad sizes heads=%d kv_heads=%d dk=%d dv=%d", heads, kv_heads, dk, dv);
   RLIS_REQUIRE(dk <= 256, "delta_scan: %d key channels, at most 256", dk);
   RLIS_REQUIRE(state_stride >= (long long)heads * dk * dv, "delta_scan: the state is too short");
   RLIS_REQUIRE(heads <= 65535 && num_seqs <= 65535, "delta_scan: grid too large");
   if (num_seqs <= 0) return 0;
-  const dim3 grid(ceil_div(dv, 4), heads, num_seqs);
+  const dim3 grid(ceil_div(dv, 4 * kCols), heads, num_seqs);
 #define LAUNCH(KR)                                                                            \
   delta_scan_kernel<KR><<<grid, 256, 0, stream>>>(out, ldo, q, k, v, ldqkv, b_raw, a_raw, ldba, \
                                                   a_log, dt_bias, state, state_stride, cu,    \
                                                   slots, heads, kv_heads, dk, dv)
-  if (dk <= 64) LAUNCH(1);
+#define LAUNCH_TILED(KR)                                                                      \
+  delta_scan_tiled_kernel<KR><<<grid, 256, 0, stream>>>(out, ldo, q, k, v, ldqkv, b_raw, a_raw, \
+                                                        ldba, a_log, dt_bias, state,          \
+                                                        state_stride, cu, slots, heads,       \
+                                                        kv_heads, dk, dv)
+  // `tiled`: some sequence of the step brings many tokens (the caller knows from the host)
+  if (tiled) {
+    if (dk <= 64) LAUNCH_TILED(1);
+    else if (dk <= 128) LAUNCH_TILED(2);
+    else LAUNCH_TILED(4);
+  } else if (dk <= 64) LAUNCH(1);
   else if (dk <= 128) LAUNCH(2);
   else LAUNCH(4);
 #undef LAUNCH
+#undef LAUNCH_TILED
   RLIS_LAUNCH_CHECK("delta_scan");
   return 0;
 }
@@ -400,7 +764,7 @@ RLIS_API int rlis_delta_scan(float* out, long long ldo, const float* q, const fl
 RLIS_API int rlis_decay_scan(float* out, const float* r, const float* k, const float* v,
                              const float* z, long long ld, const float* w0, const float* bonus,
                              float* state, long long state_stride, const int* cu,
-                             const int* slots, int num_seqs, int heads, int d,
+                             const int* slots, int num_seqs, int heads, int d, int tiled,
                              hipStream_t stream) {
   RLIS_REQUIRE(heads > 0 && d > 0 && d <= 256, "decay_scan: bad sizes heads=%d d=%d (at most 256)",
                heads, d);
@@ -408,14 +772,22 @@ RLIS_API int rlis_decay_scan(float* out, const float* r, const float* k, const f
   RLIS_REQUIRE(state_stride >= (long long)heads * d * d, "decay_scan: the state is too short");
   RLIS_REQUIRE(heads <= 65535 && num_seqs <= 65535, "decay_scan: grid too large");
   if (num_seqs <= 0) return 0;
-  const dim3 grid(ceil_div(d, 4), heads, num_seqs);
+  const dim3 grid(ceil_div(d, 4 * kCols), heads, num_seqs);
 #define LAUNCH(KR)                                                                           \
   decay_scan_kernel<KR><<<grid, 256, 0, stream>>>(out, r, k, v, z, ld, w0, bonus, state,     \
                                                   state_stride, cu, slots, heads, d)
-  if (d <= 64) LAUNCH(1);
+#define LAUNCH_TILED(KR)                                                                     \
+  decay_scan_tiled_kernel<KR><<<grid, 256, 0, stream>>>(out, r, k, v, z, ld, w0, bonus, state, \
+                                                        state_stride, cu, slots, heads, d)
+  if (tiled) {
+    if (d <= 64) LAUNCH_TILED(1);
+    else if (d <= 128) LAUNCH_TILED(2);
+    else LAUNCH_TILED(4);
+  } else if (d <= 64) LAUNCH(1);
   else if (d <= 128) LAUNCH(2);
   else LAUNCH(4);
 #undef LAUNCH
+#undef LAUNCH_TILED
   RLIS_LAUNCH_CHECK("decay_scan");
   return 0;
 }

@@ -27,8 +27,8 @@ _SIGNATURES = {
     "rlis_shift_mix": [P, P, I, P, P, L, P, P, P, I, I, I, P],
     "rlis_tail_update": [P, L, P, I, L, I, I, P, P, I, P],
     "rlis_causal_conv": [P, P, L, P, I, I, P, L, P, P, P, I, I, I, I, F, F, I, P],
-    "rlis_delta_scan": [P, L, P, P, P, L, P, P, L, P, P, P, L, P, P, I, I, I, I, I, P],
-    "rlis_decay_scan": [P, P, P, P, P, L, P, P, P, L, P, P, I, I, I, P],
+    "rlis_delta_scan": [P, L, P, P, P, L, P, P, L, P, P, P, L, P, P, I, I, I, I, I, I, P],
+    "rlis_decay_scan": [P, P, P, P, P, L, P, P, P, L, P, P, I, I, I, I, P],
     "rlis_head_norm_gate": [P, I, P, P, I, P, I, L, I, I, I, F, P],
     "rlis_rope_kv_write": [P, I, L, I, I, I, I, I, I, I, P, P, P, P, P, P, I, I, I, I, P],
     "rlis_copy_pages": [P, I, I, L, L, P, P, I, P],

@@ -8,6 +8,8 @@ cumulative token counts, state slots and sequence of each token, int32 on the de
 function checks on the host what its kernel and grid assume."""
 from __future__ import annotations
 
+from typing import Optional
+
 import torch
 
 from . import lib
@@ -51,6 +53,15 @@ def _vec(t: torch.Tensor, n: int, what: str) -> int:
         raise KernelError(f"{what}: needs {n} contiguous float32 values on the GPU, got "
                           f"{tuple(t.shape)} {t.dtype}")
     return t.data_ptr()
+
+
+# A step with at least this many tokens per sequence on average takes the scans' tiled kernels
+# (known from the host: the number of rows and of sequences).
+TILED_SCAN_MIN_MEAN_TOKENS = 4
+
+
+def _long_runs(T: int, num_seqs: int) -> bool:
+    return T >= TILED_SCAN_MIN_MEAN_TOKENS * max(1, num_seqs)
 
 
 def shift_mix(x: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, seq_of_token: torch.Tensor,
@@ -113,14 +124,18 @@ def causal_conv(x: torch.Tensor, taps: torch.Tensor, state: torch.Tensor,
 def delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, b_raw: torch.Tensor,
                a_raw: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor,
                state: torch.Tensor, cu: torch.Tensor, slots: torch.Tensor, num_seqs: int,
-               heads: int, kv_heads: int, dk: int, dv: int) -> torch.Tensor:
+               heads: int, kv_heads: int, dk: int, dv: int,
+               tiled: Optional[bool] = None) -> torch.Tensor:
     """The gated delta rule over every sequence's tokens of the step.  ``q``, ``k``
     ``(T, kv_heads * dk)`` and ``v (T, heads * dv)`` are float32 column ranges of one matrix
     (one row stride), ``b_raw``, ``a_raw`` ``(T, heads)`` of another; per token and head
     ``S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q`` with
     ``g = exp(-exp(a_log) * softplus(a_raw + dt_bias))`` and ``beta = sigmoid(b_raw)``.
     ``state (slots, heads * dv * dk)`` holds S as [head][value channel][key channel] and is
-    left as after each sequence's last token.  Returns ``o (T, heads * dv)`` float32."""
+    left as after each sequence's last token.  Returns ``o (T, heads * dv)`` float32.
+    ``tiled`` chooses the kernel that stages tiles of tokens through LDS (for steps in which a
+    sequence brings many tokens; None: from four tokens per sequence on average); the two
+    agree to rounding (the tiled kernel forms a token's four sums over the wave together)."""
     ld = _rows(q, "delta_scan q", torch.float32)
     if _rows(k, "delta_scan k", torch.float32) != ld or _rows(v, "delta_scan v", torch.float32) != ld:
         raise KernelError("delta_scan: q, k and v must share a row stride")
@@ -137,18 +152,20 @@ def delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, b_raw: torch.T
              v.data_ptr(), ld, b_raw.data_ptr(), a_raw.data_ptr(), ldba,
              _vec(a_log, heads, "delta_scan A_log"), _vec(dt_bias, heads, "delta_scan dt_bias"),
              state.data_ptr(), stride, _meta(cu, num_seqs + 1, "cu"),
-             _meta(slots, num_seqs, "slots"), num_seqs, heads, kv_heads, dk, dv, lib.stream_ptr())
+             _meta(slots, num_seqs, "slots"), num_seqs, heads, kv_heads, dk, dv,
+             int(_long_runs(T, num_seqs) if tiled is None else bool(tiled)), lib.stream_ptr())
     return out
 
 
 def decay_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch.Tensor,
                w0: torch.Tensor, bonus: torch.Tensor, state: torch.Tensor, cu: torch.Tensor,
-               slots: torch.Tensor, num_seqs: int, heads: int, d: int) -> torch.Tensor:
+               slots: torch.Tensor, num_seqs: int, heads: int, d: int,
+               tiled: Optional[bool] = None) -> torch.Tensor:
     """A matrix state per head with a decay per key channel and a bonus for the current token:
     per token ``o = (S + diag(bonus) k v^T)^T r; S <- diag(w) S + k v^T`` with
     ``w = exp(-exp(z + w0))``.  ``r``, ``k``, ``v``, ``z`` are contiguous float32
     ``(T, heads * d)``; ``state (slots, heads * d * d)`` holds S as [head][value channel][key
-    channel].  Returns ``o (T, heads * d)`` float32."""
+    channel].  Returns ``o (T, heads * d)`` float32.  ``tiled`` as for ``delta_scan``."""
     T = r.shape[0]
     for name, t in (("r", r), ("k", k), ("v", v), ("z", z)):
         if not t.is_cuda or t.dtype != torch.float32 or t.shape != (T, heads * d) \
@@ -160,7 +177,7 @@ def decay_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch.Tenso
              z.data_ptr(), heads * d, _vec(w0, heads * d, "decay_scan w0"),
              _vec(bonus.reshape(-1), heads * d, "decay_scan bonus"), state.data_ptr(), stride,
              _meta(cu, num_seqs + 1, "cu"), _meta(slots, num_seqs, "slots"), num_seqs, heads, d,
-             lib.stream_ptr())
+             int(_long_runs(T, num_seqs) if tiled is None else bool(tiled)), lib.stream_ptr())
     return out
 
 

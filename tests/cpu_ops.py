@@ -97,7 +97,7 @@ def causal_conv(x, taps, state, seq_of_token, cu, slots, num_seqs, unit_channels
 
 
 def delta_scan(q, k, v, b_raw, a_raw, a_log, dt_bias, state, cu, slots, num_seqs, heads,
-               kv_heads, dk, dv):
+               kv_heads, dk, dv, tiled=None):
     T = q.shape[0]
     out = torch.empty((T, heads * dv), dtype=torch.float32)
     g = torch.exp(-torch.exp(a_log) * torch.nn.functional.softplus(a_raw + dt_bias))
@@ -116,7 +116,7 @@ def delta_scan(q, k, v, b_raw, a_raw, a_log, dt_bias, state, cu, slots, num_seqs
     return out
 
 
-def decay_scan(r, k, v, z, w0, bonus, state, cu, slots, num_seqs, heads, d):
+def decay_scan(r, k, v, z, w0, bonus, state, cu, slots, num_seqs, heads, d, tiled=None):
     T = r.shape[0]
     out = torch.empty((T, heads * d), dtype=torch.float32)
     w = torch.exp(-torch.exp(z + w0)).reshape(T, heads, d)

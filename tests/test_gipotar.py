@@ -225,7 +225,7 @@ def test_a_far_key_that_stands_out(backend, dtype, far, tmp_path_factory):
     for name, token in (("l0.mix.left.k", key_token), ("l0.mix.left.q", query_token)):
         direction = w["embed"][token] / w["embed"][token].norm()
         for head in range(left["heads"] if name.endswith("q") else left["kv_heads"]):
-            w[name][head * d:(head + 1) * d] += 6.0 * torch.outer(probe, direction)
+            w[name][head * d:(head + 1) * d] += 0.25 * torch.outer(probe, direction)
     folder, _, stored = model_case("b", dtype, tmp_path_factory, weights=w, tag=f"far")
     tokens = [t if t not in (key_token, query_token) else 1
               for t in gm.prompts(cfg["vocab"], [100], seed=22)[0]]

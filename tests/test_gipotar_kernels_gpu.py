@@ -31,7 +31,8 @@ def _state(num_slots, used, extra=24):
     return buf, buf[:, 8:8 + used]
 
 
-STEPS = [[5, 1, 9], [1, 1, 2], [3, 1, 1], [17, 2, 1]]      # tokens per sequence, step by step
+# tokens per sequence, step by step (a run longer than a tile of the tiled scans among them)
+STEPS = [[5, 1, 9], [1, 1, 2], [3, 1, 1], [17, 2, 1], [2, 70, 33]]
 SLOTS = [3, 0, 2]
 
 
@@ -41,8 +42,11 @@ def _cut(x, lengths_by_step, step, seq):
     return slice(start, start + lengths_by_step[step][seq])
 
 
+@pytest.mark.parametrize("tiled", [False, True, None])
 @pytest.mark.parametrize("heads, d", [(3, 16), (2, 96), (1, 160), (2, 50)])
-def test_decayed_state_scan(heads, d):
+def test_decayed_state_scan(heads, d, tiled):
+    """``tiled``: the kernel that stages tiles of tokens through LDS, the one that asks for a
+    token's vectors one token ahead, or whichever the step's shape chooses."""
     ops = _ops()
     g = torch.Generator().manual_seed(heads * 100 + d)
     totals = [sum(s[i] for s in STEPS) for i in range(3)]
@@ -63,7 +67,7 @@ def test_decayed_state_scan(heads, d):
         rows = {n: torch.cat([data[i][n][_cut(None, STEPS, step, i)] for i in range(3)]).to(DEV)
                 for n in "rkvz"}
         out = ops.decay_scan(rows["r"], rows["k"], rows["v"], rows["z"], w0.to(DEV),
-                             bonus.to(DEV), state, cu, slots, 3, heads, d).cpu()
+                             bonus.to(DEV), state, cu, slots, 3, heads, d, tiled=tiled).cpu()
         at = 0
         for i, n in enumerate(lengths):
             ref = want[i][_cut(None, STEPS, step, i)].reshape(n, heads * d)
@@ -75,9 +79,10 @@ def test_decayed_state_scan(heads, d):
     assert float(buf[1].min()) == 7.5 and float(buf[:, :8].min()) == 7.5     # nothing else moved
 
 
+@pytest.mark.parametrize("tiled", [False, True, None])
 @pytest.mark.parametrize("heads, groups, dk, dv", [(4, 2, 16, 24), (2, 1, 96, 6), (1, 1, 200, 33),
                                                    (6, 3, 64, 64)])
-def test_gated_delta_scan(heads, groups, dk, dv):
+def test_gated_delta_scan(heads, groups, dk, dv, tiled):
     ops = _ops()
     g = torch.Generator().manual_seed(dk * 10 + dv)
     totals = [sum(s[i] for s in STEPS) for i in range(3)]
@@ -109,7 +114,7 @@ def test_gated_delta_scan(heads, groups, dk, dv):
         out = ops.delta_scan(qkv[:, :groups * dk], qkv[:, groups * dk:2 * groups * dk],
                              qkv[:, 2 * groups * dk:], ba[:, :heads], ba[:, heads:],
                              a_log.to(DEV), dt_bias.to(DEV), state, cu, slots, 3, heads, groups,
-                             dk, dv).cpu()
+                             dk, dv, tiled=tiled).cpu()
         at = 0
         for i, n in enumerate(lengths):
             ref = want[i][_cut(None, STEPS, step, i)].reshape(n, heads * dv)
