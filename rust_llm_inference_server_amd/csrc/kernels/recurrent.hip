@@ -34,16 +34,18 @@ __global__ void shift_mix_kernel(TX* __restrict__ out, const TX* __restrict__ x,
                                  const int* __restrict__ cu, const int* __restrict__ slots, int T,
                                  int W, int mixes) {
   const int t = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= W) return;
   const int s = seq_of_token[t];
   const bool first = t == cu[s];
   const float* tail = state + (long long)slots[s] * state_stride;
-  for (int c = threadIdx.x; c < W; c += blockDim.x) {
-    const float cur = ld(x + (long long)t * W + c);
-    const float prev = first ? tail[c] : ld(x + (long long)(t - 1) * W + c);
-    const float d = prev - cur;
-    for (int m = 0; m < mixes; ++m)
-      st(out + ((long long)m * T + t) * W + c, cur + d * mu[(long long)m * W + c]);
-  }
+  // both candidates are asked for, from addresses that always exist, and the value is chosen
+  const float cur = ld(x + (long long)t * W + c);
+  const float before = ld(x + (long long)(t > 0 ? t - 1 : 0) * W + c);
+  const float kept = tail[c];
+  const float d = (first ? kept : before) - cur;
+  for (int m = 0; m < mixes; ++m)
+    st(out + ((long long)m * T + t) * W + c, cur + d * mu[(long long)m * W + c]);
 }
 
 // ------------------------------------------------------------------ input tails
@@ -664,13 +666,15 @@ RLIS_API int rlis_shift_mix(void* out, const void* x, int dtype, const float* mu
                             hipStream_t stream) {
   RLIS_REQUIRE(T >= 0 && W > 0 && mixes > 0, "shift_mix: bad sizes T=%d W=%d mixes=%d", T, W, mixes);
   RLIS_REQUIRE(state_stride >= W, "shift_mix: the state is shorter than a row");
+  RLIS_REQUIRE(ceil_div(W, 256) <= 65535, "shift_mix: W=%d is too wide", W);
   if (T == 0) return 0;
+  const dim3 grid(T, ceil_div(W, 256));
   if (dtype == RLIS_F32)
-    shift_mix_kernel<float><<<T, 256, 0, stream>>>((float*)out, (const float*)x, mu, state,
+    shift_mix_kernel<float><<<grid, 256, 0, stream>>>((float*)out, (const float*)x, mu, state,
                                                    state_stride, seq_of_token, cu, slots, T, W,
                                                    mixes);
   else if (dtype == RLIS_BF16)
-    shift_mix_kernel<bf16_t><<<T, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)x, mu, state,
+    shift_mix_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)x, mu, state,
                                                     state_stride, seq_of_token, cu, slots, T, W,
                                                     mixes);
   else

@@ -54,6 +54,7 @@ class ClampedGLU(FeedForward):
     ``gate_proj.weight`` and so on)."""
 
     graph_safe = True
+    takes_normed_input = True        # the norm in front goes into the gate/up product where it can
 
     _DEFAULT_NAMES = {"gate": "gate_proj.weight", "up": "up_proj.weight",
                       "down": "down_proj.weight"}
@@ -86,6 +87,6 @@ class ClampedGLU(FeedForward):
         self.act_dtype = ctx.act_dtype
 
     def forward(self, x: Any, step: Any) -> torch.Tensor:
-        gu = ops.linear(x, self.w_gate_up, self.act_dtype)
+        gu = project(x, self.w_gate_up, self.act_dtype)
         hidden = ops.clamped_glu(gu, self.limit, self.alpha)
         return ops.pending_linear(hidden, self.w_down, self.act_dtype)

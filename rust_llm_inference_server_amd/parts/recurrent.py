@@ -28,7 +28,7 @@ import torch
 
 from .. import ops
 from .base import (BuildContext, CacheBinding, CacheRequest, Mixer, PartSpec, TensorSpec,
-                   as_tensor, create, join, register, tensor_specs)
+                   as_tensor, create, join, project, register, tensor_specs)
 
 
 def _f32(t: torch.Tensor) -> torch.Tensor:
@@ -126,6 +126,7 @@ class GatedDelta(Mixer):
     part starting on a multiple of 8 columns), stored in float32."""
 
     graph_safe = True
+    takes_normed_input = True        # the norm in front goes into the one input product where it can
     UNIT_EPS = 1e-6
 
     @classmethod
@@ -184,11 +185,11 @@ class GatedDelta(Mixer):
     def state_bytes(self) -> int:
         return 4 * ((self.taps - 1) * self.conv_channels + self.heads * self.vdim * self.dim)
 
-    def forward(self, x: torch.Tensor, step: Any, binding: CacheBinding) -> Any:
+    def forward(self, x: Any, step: Any, binding: CacheBinding) -> Any:
         G, H, d, dv, C = self.kv_heads, self.heads, self.dim, self.vdim, self.conv_channels
         tail, S = _state_views(binding, (self.taps - 1) * C)
         cu, slots, n = step.cu_seqlens, step.state_slots, step.num_seqs
-        p = ops.linear(x, self.w_in, torch.float32)                       # (T, q|k|v|g|b|a)
+        p = project(x, self.w_in, torch.float32)                          # (T, q|k|v|g|b|a)
         qkv = ops.causal_conv(p, self.conv_w, tail, step.seq_of_token, cu, slots, n,
                               unit_channels=2 * G * d, unit_group=d, scaled_channels=G * d,
                               scale=d ** -0.5, unit_eps=self.UNIT_EPS, rest_group=dv)
