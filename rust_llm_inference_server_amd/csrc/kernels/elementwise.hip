@@ -530,24 +530,35 @@ RLIS_API int rlis_clamped_glu(void* out, const void* gu, int dtype, int T, int I
 
 // ------------------------------------------------------------- weighted sum of two
 // out (float32) = a * x + b * y, element by element: two branches that read the same input
-// meet here on their way into the residual stream.
+// meet here on their way into the residual stream.  Either operand may come as a stack of
+// float32 partial sums, n elements apart, which are added in order first (and, with round16,
+// rounded to bfloat16 as a result that arrives whole in bfloat16 was); y may be absent.
 template <typename TX, typename TY>
 __global__ void weighted_sum_kernel(float* __restrict__ out, const TX* __restrict__ x, float a,
-                                    const TY* __restrict__ y, float b, long long n) {
+                                    int x_parts, const TY* __restrict__ y, float b, int y_parts,
+                                    long long n, int round16) {
   long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   const long long stride = (long long)gridDim.x * blockDim.x;
-  for (; i < n; i += stride) out[i] = a * ld(x + i) + b * ld(y + i);
+  for (; i < n; i += stride) {
+    float v = a * delta_sum(x + i, x_parts, n, round16 && x_parts > 1);
+    if (y) v += b * delta_sum(y + i, y_parts, n, round16 && y_parts > 1);
+    out[i] = v;
+  }
 }
 
-RLIS_API int rlis_weighted_sum(float* out, const void* x, int x_dtype, float a, const void* y,
-                               int y_dtype, float b, long long n, hipStream_t stream) {
+RLIS_API int rlis_weighted_sum(float* out, const void* x, int x_dtype, float a, int x_parts,
+                               const void* y, int y_dtype, float b, int y_parts, long long n,
+                               int round16, hipStream_t stream) {
+  RLIS_REQUIRE(x && x_parts >= 1 && (!y || y_parts >= 1), "weighted_sum: bad operands");
+  RLIS_REQUIRE((x_parts == 1 || x_dtype == RLIS_F32) && (!y || y_parts == 1 || y_dtype == RLIS_F32),
+               "weighted_sum: partial sums are float32");
   if (n <= 0) return 0;
   const int blocks = (int)(ceil_div_ll(n, 256) < 8192 ? ceil_div_ll(n, 256) : 8192);
-  const int key = x_dtype * 2 + y_dtype;
-#define CASE(k, TX, TY)                                                                       \
-  case k:                                                                                     \
-    weighted_sum_kernel<TX, TY><<<blocks, 256, 0, stream>>>(out, (const TX*)x, a, (const TY*)y, \
-                                                            b, n);                            \
+  const int key = x_dtype * 2 + (y ? y_dtype : 0);
+#define CASE(k, TX, TY)                                                                        \
+  case k:                                                                                      \
+    weighted_sum_kernel<TX, TY><<<blocks, 256, 0, stream>>>(out, (const TX*)x, a, x_parts,     \
+                                                            (const TY*)y, b, y_parts, n, round16); \
     break;
   switch (key) {
     CASE(0, float, float)

@@ -269,17 +269,48 @@ def clamped_glu(gu: torch.Tensor, limit: float, alpha: float) -> torch.Tensor:
     return out
 
 
-def weighted_sum(x: torch.Tensor, a: float, y: torch.Tensor, b: float) -> torch.Tensor:
-    """``a * x + b * y`` in float32, for two tensors of one shape (float32 or bfloat16 each)."""
-    _check(x, "weighted_sum x")
-    _check(y, "weighted_sum y")
-    if x.shape != y.shape or not x.is_contiguous() or not y.is_contiguous():
-        raise KernelError(f"weighted_sum: contiguous tensors of one shape, got {tuple(x.shape)} "
-                          f"and {tuple(y.shape)}")
-    out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
-    lib.call("rlis_weighted_sum", out.data_ptr(), x.data_ptr(), _dt(x), float(a), y.data_ptr(),
-             _dt(y), float(b), x.numel(), lib.stream_ptr())
+def _whole_or_parts(t: torch.Tensor, what: str) -> Tuple[int, Tuple[int, ...]]:
+    """(parts, shape of the whole) of a tensor that is whole, or a stack of float32 partial sums
+    along a leading axis (what ``linear(..., partials=True)`` may return)."""
+    _check(t, what)
+    if not t.is_contiguous():
+        raise KernelError(f"{what}: must be contiguous")
+    if t.dim() == 3:
+        if t.dtype != torch.float32:
+            raise KernelError(f"{what}: a stack of partial sums is float32")
+        return t.shape[0], tuple(t.shape[1:])
+    return 1, tuple(t.shape)
+
+
+def weighted_sum(x: torch.Tensor, a: float, y: Optional[torch.Tensor], b: float = 0.0,
+                 round_parts: bool = False) -> torch.Tensor:
+    """``a * x + b * y`` in float32 for two ``(T, N)`` tensors (float32 or bfloat16 each); either
+    may be a stack ``(S, T, N)`` of float32 partial sums, added in order first (and with
+    ``round_parts`` rounded to bfloat16, as a result that arrives whole in bfloat16 was).
+    ``y`` None: ``a * x``."""
+    x_parts, shape = _whole_or_parts(x, "weighted_sum x")
+    y_parts = 1
+    if y is not None:
+        y_parts, y_shape = _whole_or_parts(y, "weighted_sum y")
+        if y_shape != shape:
+            raise KernelError(f"weighted_sum: shapes {shape} and {y_shape} differ")
+    out = torch.empty(shape, dtype=torch.float32, device=x.device)
+    lib.call("rlis_weighted_sum", out.data_ptr(), x.data_ptr(), _dt(x), float(a), x_parts,
+             None if y is None else y.data_ptr(), 0 if y is None else _dt(y), float(b), y_parts,
+             out.numel(), int(bool(round_parts)), lib.stream_ptr())
     return out
+
+
+def linear_f32(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """``x @ w.T`` stored in float32, for results that enter a recurrence.  From 17 to 64 rows of
+    bfloat16 it is the split-k kernel's partial sums added in order (the library's products with
+    a float32 result are slow at such row counts: 25 us against 6 + 3 for 64 x 2,048 x 2,048);
+    otherwise ``linear(x, w, float32)``."""
+    if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 \
+            and STREAM_MAX_ROWS < x.shape[0] <= SPLITK_MAX_ROWS and x.shape[0] > stream_rows(x.shape[1]):
+        y = linear(x, w, torch.float32, partials=True)
+        return weighted_sum(y, 1.0, None) if y.dim() == 3 else y
+    return linear(x, w, torch.float32)
 
 
 def soft_cap_(x: torch.Tensor, cap: float) -> torch.Tensor:

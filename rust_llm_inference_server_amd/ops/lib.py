@@ -22,7 +22,7 @@ _SIGNATURES = {
     "rlis_add_rmsnorm": [P, P, I, P, I, P, I, P, I, I, F, I, I, L, I, F, P],
     "rlis_swiglu": [P, P, I, I, I, P],
     "rlis_clamped_glu": [P, P, I, I, I, F, F, P],
-    "rlis_weighted_sum": [P, P, I, F, P, I, F, L, P],
+    "rlis_weighted_sum": [P, P, I, F, I, P, I, F, I, L, I, P],
     "rlis_soft_cap": [P, I, L, F, P],
     "rlis_shift_mix": [P, P, I, P, P, L, P, P, P, I, I, I, P],
     "rlis_tail_update": [P, L, P, I, L, I, I, P, P, I, P],

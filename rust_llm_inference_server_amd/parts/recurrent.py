@@ -27,8 +27,8 @@ from typing import Any, Dict, List, Optional
 import torch
 
 from .. import ops
-from .base import (BuildContext, CacheBinding, CacheRequest, Mixer, PartSpec, TensorSpec,
-                   as_tensor, create, join, project, register, tensor_specs)
+from .base import (BuildContext, CacheBinding, CacheRequest, Mixer, NormedInput, PartSpec,
+                   TensorSpec, create, join, project, register, tensor_specs)
 
 
 def _f32(t: torch.Tensor) -> torch.Tensor:
@@ -43,12 +43,10 @@ def _state_views(binding: CacheBinding, first: int):
     return st[:, :first], st[:, first:]
 
 
-def _whole(delta: Any) -> torch.Tensor:
-    """A mixer's result as one ``(T, H)`` tensor; a projection that has not run yet runs as one
-    product."""
-    if isinstance(delta, ops.PendingProduct):
-        return ops.linear(delta.x, delta.w, delta.out_dtype)
-    return as_tensor(delta)
+def _ran(delta: Any) -> torch.Tensor:
+    """A mixer's result as a tensor, whole or as a stack of float32 partial sums; a projection
+    that has not run yet runs now."""
+    return delta if isinstance(delta, torch.Tensor) else delta.run()
 
 
 # ------------------------------------------------------------------------------ time mix
@@ -100,10 +98,10 @@ class TimeMix(Mixer):
         mixes = ops.shift_mix(x, self.mu, tail, step.seq_of_token, cu, slots, n)
         ops.tail_update(tail, x, self.width, 1, cu, slots, n)
         f32 = torch.float32
-        r = ops.linear(mixes[0], self.w_r, f32)
-        k = ops.linear(mixes[1], self.w_k, f32)
-        v = ops.linear(mixes[2], self.w_v, f32)
-        gate = ops.linear(mixes[3], self.w_g, f32)
+        r = ops.linear_f32(mixes[0], self.w_r)
+        k = ops.linear_f32(mixes[1], self.w_k)
+        v = ops.linear_f32(mixes[2], self.w_v)
+        gate = ops.linear_f32(mixes[3], self.w_g)
         low = ops.soft_cap_(ops.linear(mixes[4], self.w_1, self.act_dtype), 1.0)     # tanh
         z = ops.linear(low, self.w_2, f32)
         o = ops.decay_scan(r, k, v, z, self.w0, self.bonus, S, cu, slots, n, self.heads, self.dim)
@@ -189,7 +187,11 @@ class GatedDelta(Mixer):
         G, H, d, dv, C = self.kv_heads, self.heads, self.dim, self.vdim, self.conv_channels
         tail, S = _state_views(binding, (self.taps - 1) * C)
         cu, slots, n = step.cu_seqlens, step.state_slots, step.num_seqs
-        p = project(x, self.w_in, torch.float32)                          # (T, q|k|v|g|b|a)
+        if isinstance(x, NormedInput) and not ops.can_fuse_norm_linear(
+                x.stream.x, self.w_in, x.stream.x.shape[0]):
+            x = x.tensor()
+        p = (project(x, self.w_in, torch.float32) if isinstance(x, NormedInput)
+             else ops.linear_f32(x, self.w_in))                           # (T, q|k|v|g|b|a)
         qkv = ops.causal_conv(p, self.conv_w, tail, step.seq_of_token, cu, slots, n,
                               unit_channels=2 * G * d, unit_group=d, scaled_channels=G * d,
                               scale=d ** -0.5, unit_eps=self.UNIT_EPS, rest_group=dv)
@@ -265,5 +267,6 @@ class ParallelMixers(Mixer):
                 if binding.state is None:
                     raise ValueError("parallel mixer: a branch needs state, the runner has none")
                 own.state = binding.state[:, at:at + n]
-            outs.append(_whole(m.forward(x, step, own)))
-        return ops.weighted_sum(outs[0], self.scales[0], outs[1], self.scales[1])
+            outs.append(_ran(m.forward(x, step, own)))
+        return ops.weighted_sum(outs[0], self.scales[0], outs[1], self.scales[1],
+                                round_parts=x.dtype == torch.bfloat16)

@@ -44,8 +44,16 @@ def clamped_glu(gu, limit, alpha):
     return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gu.dtype)
 
 
-def weighted_sum(x, a, y, b):
-    return a * x.float() + b * y.float()
+def weighted_sum(x, a, y, b=0.0, round_parts=False):
+    x = x.sum(0) if x.dim() == 3 else x
+    out = a * x.float()
+    if y is not None:
+        out = out + b * (y.sum(0) if y.dim() == 3 else y).float()
+    return out
+
+
+def linear_f32(x, w):
+    return linear(x, w, torch.float32)
 
 
 def soft_cap_(x, cap):
@@ -260,7 +268,7 @@ def install(monkeypatch) -> None:
     for name in ("embed", "add_residual", "add_rmsnorm", "swiglu", "linear", "linear_swiglu",
                  "pending_linear", "can_fuse_norm_linear", "rope_kv_write", "rope_attention",
                  "copy_pages", "attention_planner", "paged_attention", "sample_rows",
-                 "clamped_glu", "weighted_sum", "soft_cap_", "shift_mix", "tail_update",
+                 "clamped_glu", "weighted_sum", "linear_f32", "soft_cap_", "shift_mix", "tail_update",
                  "causal_conv", "delta_scan", "decay_scan", "head_norm_gate"):
         monkeypatch.setattr(ops, name, globals()[name])
     monkeypatch.setattr(runner, "default_device", lambda: torch.device("cpu"))

@@ -213,6 +213,19 @@ def test_clamped_gated_unit_weighted_sum_and_caps():
     x, y = torch.randn(7, 33, generator=g), torch.randn(7, 33, generator=g).to(torch.bfloat16)
     got = ops.weighted_sum(x.to(DEV), 0.8, y.to(DEV), -0.5).cpu().double()
     assert torch.allclose(got, 0.8 * x.double() - 0.5 * y.double(), atol=1e-6)
+    # stacks of partial sums on either side, added in order (and rounded once when asked)
+    xs, ys = torch.randn(3, 7, 33, generator=g), torch.randn(5, 7, 33, generator=g)
+    got = ops.weighted_sum(xs.to(DEV), 1.5, ys.to(DEV), 0.25).cpu().double()
+    assert torch.allclose(got, 1.5 * xs.double().sum(0) + 0.25 * ys.double().sum(0), atol=1e-5)
+    got = ops.weighted_sum(xs.to(DEV), 1.0, None, round_parts=True).cpu()
+    assert torch.equal(got, ((xs[0] + xs[1]) + xs[2]).to(torch.bfloat16).float())
+    # a float32 result from bfloat16 operands at every row count's kernel
+    w = (torch.randn(96, 512, generator=g) * 0.05).to(torch.bfloat16)
+    for rows in (1, 16, 17, 40, 64, 65, 200):
+        xr = torch.randn(rows, 512, generator=g).to(torch.bfloat16)
+        got = ops.linear_f32(xr.to(DEV), w.to(DEV)).cpu()
+        assert got.dtype == torch.float32 and got.shape == (rows, 96)
+        assert torch.allclose(got.double(), xr.double() @ w.double().T, rtol=1e-4, atol=1e-4)
     z = torch.randn(5, 19, generator=g) * 40.0
     assert torch.allclose(ops.soft_cap_(z.clone().to(DEV), 30.0).cpu().double(),
                           30.0 * torch.tanh(z.double() / 30.0), atol=1e-5)
