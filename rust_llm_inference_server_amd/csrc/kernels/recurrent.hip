@@ -80,17 +80,22 @@ __global__ void tail_update_kernel(float* __restrict__ state, long long state_st
 // the tail, rows in front of the sequence are the tail's zeros.  Channels [0, unit_channels)
 // are then made unit vectors in groups of unit_group (x / sqrt(sum x^2 + unit_eps)) and those
 // below scaled_channels multiplied by `scale`; the other channels are cut into groups of
-// rest_group for the grid only.  One block per (token, group), up to 4 channels per thread.
+// rest_group for the grid only.  One wave per (token, group), up to 16 channels per lane; a
+// workgroup is four groups of one token.  Both candidates of an input row (the step's, the
+// tail's) are asked for from addresses that exist, and the value is chosen.
+__device__ __forceinline__ float lanes_sum(float v);
+
 __global__ __launch_bounds__(256) void causal_conv_kernel(
     float* __restrict__ out, const float* __restrict__ x, long long ldx,
     const float* __restrict__ taps, int C, int K, const float* __restrict__ state,
     long long state_stride, const int* __restrict__ seq_of_token, const int* __restrict__ cu,
     const int* __restrict__ slots, int unit_channels, int unit_group, int scaled_channels,
-    float scale, float unit_eps, int rest_group) {
-  __shared__ float red[256 / kWave];
+    float scale, float unit_eps, int rest_group, int groups) {
   const int t = blockIdx.x;
+  const int lane = threadIdx.x % kWave;
+  const int g = blockIdx.y * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (g >= groups) return;
   const int groups_unit = unit_group > 0 ? unit_channels / unit_group : 0;
-  const int g = blockIdx.y;
   int c0, width;
   const bool unit = g < groups_unit;
   if (unit) {
@@ -104,34 +109,37 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(
   const int rel = t - cu[s];                 // rows of the step in front of this one
   const int R = K - 1;
   const float* tail = state + (long long)slots[s] * state_stride;
-  float y[4];
+  constexpr int VPT = 16;
+  float y[VPT];
   float ss = 0.f;
 #pragma unroll
-  for (int v = 0; v < 4; ++v) {
-    const int c = c0 + threadIdx.x + v * 256;
+  for (int v = 0; v < VPT; ++v) {
     y[v] = 0.f;
-    if (threadIdx.x + v * 256 < width) {
+    if (v * kWave < width) {                 // the same for the whole wave
+      const int off = lane + v * kWave;
+      const int c = c0 + (off < width ? off : width - 1);
       float acc = 0.f;
       for (int j = 0; j < K; ++j) {
         const int back = R - j;              // how many rows before t
-        const float in = back <= rel ? x[(long long)(t - back) * ldx + c]
-                                     : tail[(long long)(R - (back - rel)) * C + c];
-        acc += taps[(long long)c * K + j] * in;
+        const bool here = back <= rel;
+        const float from_step = x[(long long)(t - (here ? back : 0)) * ldx + c];
+        const float from_tail = R > 0 ? tail[(long long)(here ? 0 : R - (back - rel)) * C + c] : 0.f;
+        acc += taps[(long long)c * K + j] * (here ? from_step : from_tail);
       }
-      y[v] = siluf_(acc);
+      y[v] = off < width ? siluf_(acc) : 0.f;
       ss += y[v] * y[v];
     }
   }
   float mult = 1.0f;
   if (unit) {
-    ss = block_sum<256>(ss, red);
+    ss = lanes_sum(ss);
     mult = 1.0f / sqrtf(ss + unit_eps);
     if (c0 < scaled_channels) mult *= scale;
   }
 #pragma unroll
-  for (int v = 0; v < 4; ++v) {
-    const int c = c0 + threadIdx.x + v * 256;
-    if (threadIdx.x + v * 256 < width) out[(long long)t * C + c] = y[v] * mult;
+  for (int v = 0; v < VPT; ++v) {
+    const int off = lane + v * kWave;
+    if (off < width) out[(long long)t * C + c0 + off] = y[v] * mult;
   }
 }
 
@@ -143,7 +151,7 @@ template <int CTRL>
 __device__ __forceinline__ float dpp_from(float v) {
   return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
 }
-__device__ __forceinline__ float lanes_sum(float v) {
+__device__ __forceinline__ float lanes_sum(float v) {   // (declared above, for the convolution)
   v += dpp_from<0xB1>(v);    // quad_perm [1, 0, 3, 2]
   v += dpp_from<0x4E>(v);    // quad_perm [2, 3, 0, 1]
   v += dpp_from<0x141>(v);   // row_half_mirror
@@ -721,10 +729,10 @@ RLIS_API int rlis_causal_conv(float* out, const float* x, long long ldx, const f
   if (T == 0) return 0;
   const int groups = (unit_channels ? unit_channels / unit_group : 0) +
                      (unit_channels < C ? ceil_div(C - unit_channels, rest_group) : 0);
-  RLIS_REQUIRE(groups <= 65535, "causal_conv: too many groups");
-  causal_conv_kernel<<<dim3(T, groups), 256, 0, stream>>>(
+  RLIS_REQUIRE(ceil_div(groups, 4) <= 65535, "causal_conv: too many groups");
+  causal_conv_kernel<<<dim3(T, ceil_div(groups, 4)), 256, 0, stream>>>(
       out, x, ldx, taps, C, K, state, state_stride, seq_of_token, cu, slots, unit_channels,
-      unit_group, scaled_channels, scale, unit_eps, rest_group > 0 ? rest_group : 1);
+      unit_group, scaled_channels, scale, unit_eps, rest_group > 0 ? rest_group : 1, groups);
   RLIS_LAUNCH_CHECK("causal_conv");
   return 0;
 }

@@ -210,6 +210,10 @@ def test_clamped_gated_unit_weighted_sum_and_caps():
     got = ops.clamped_glu(gu.to(DEV), 1.5, 1.702).cpu().double()
     gate, up = gu[:, :37].double().clamp(max=1.5), gu[:, 37:].double().clamp(-1.5, 1.5)
     assert torch.allclose(got, gate * torch.sigmoid(1.702 * gate) * (up + 1.0), atol=1e-6)
+    gu16 = (torch.randn(9, 2 * 48, generator=g) * 3.0).to(torch.bfloat16)     # 16-byte form
+    got = ops.clamped_glu(gu16.to(DEV), 2.0, 1.702).cpu().double()
+    gate, up = gu16[:, :48].double().clamp(max=2.0), gu16[:, 48:].double().clamp(-2.0, 2.0)
+    assert torch.allclose(got, gate * torch.sigmoid(1.702 * gate) * (up + 1.0), rtol=1e-2, atol=1e-2)
     x, y = torch.randn(7, 33, generator=g), torch.randn(7, 33, generator=g).to(torch.bfloat16)
     got = ops.weighted_sum(x.to(DEV), 0.8, y.to(DEV), -0.5).cpu().double()
     assert torch.allclose(got, 0.8 * x.double() - 0.5 * y.double(), atol=1e-6)
