@@ -54,7 +54,26 @@ CONFIG_B = {
         _parallel(_attn(4, 1, 16, 16, 4, 200.0, 0.4), 4, 16, 4, 0.5, 0.9, None),
     ],
 }
-CONFIGS = {"a": CONFIG_A, "b": CONFIG_B}
+# Only the delta rule (no mixer asks for pages), one layer with a single tap (no tail at all)
+# and one whose three value heads share one query/key head; and only parallel layers, one with
+# no rotation and heads of 24 (no multiple of 16: the generic attention kernel in bfloat16).
+CONFIG_C = {
+    "architecture": "Gipotar", "vocab": 64, "width": 40, "embedding": {"scale": 2.0},
+    "residual_mult": 0.8, "norm": {"eps": 1e-5}, "logit_softcap": 20.0,
+    "layers": [
+        _delta(2, 2, 24, 16, 1, None),
+        _delta(3, 1, 16, 24, 4, _mlp(48, 2.0)),
+    ],
+}
+CONFIG_D = {
+    "architecture": "Gipotar", "vocab": 80, "width": 48, "embedding": {"scale": 4.0},
+    "residual_mult": 0.9, "norm": {"eps": 1e-6}, "logit_softcap": 15.0,
+    "layers": [
+        _parallel(_attn(2, 2, 24, 24, 0, 10000.0, 0.2), 2, 16, 8, 0.6, 0.8, _mlp(64, 2.0)),
+        _parallel(_attn(3, 1, 16, 48, 16, 300.0, 0.25), 1, 32, 3, 1.2, 0.3, None),
+    ],
+}
+CONFIGS = {"a": CONFIG_A, "b": CONFIG_B, "c": CONFIG_C, "d": CONFIG_D}
 
 
 def spec_of(config: dict):
