@@ -199,6 +199,33 @@ def test_a_request_alone_equals_itself_in_a_batch(backend, dtype, tmp_path_facto
               for pos, row in together[rid].items()], dtype)
 
 
+@pytest.mark.parametrize("live", [20, 40])
+def test_decode_steps_of_many_requests(backend, dtype, live, tmp_path_factory):
+    """Twenty and forty requests decoding together (the products' kernels for 17 to 32 and for
+    33 to 64 rows, their float32 results from partial sums, captured steps of those sizes), each
+    row against its request's plain logits; prompts of unequal length arrive in two steps."""
+    from rust_llm_inference_server_amd.engine import StepEntry
+    folder, cfg, stored = model_case("a", dtype, tmp_path_factory)
+    if backend.type == "cpu" and live > 20:
+        pytest.skip("the double has one kernel for every row count")
+    prompts = gm.prompts(cfg["vocab"], [3 + (7 * i) % 23 for i in range(live)], seed=23)
+    new = 5
+    tails = gm.prompts(cfg["vocab"], [new] * live, seed=24)
+    runner = runner_for(folder, backend, dtype, num_pages=4 * live, max_num_seqs=live)
+    errors = []
+    want = [plain.forward(cfg, stored, p + t) for p, t in zip(prompts, tails)]
+    for lo, hi in ((0, live // 2), (live // 2, live)):
+        for i in range(lo, hi):
+            runner.reserve(i, len(prompts[i]) + new)
+        out = runner.step([StepEntry(i, prompts[i], [len(prompts[i]) - 1]) for i in range(lo, hi)])
+        errors += [gm.row_error(out[j].cpu(), want[i][len(prompts[i]) - 1])
+                   for j, i in enumerate(range(lo, hi))]
+    for k in range(new):
+        out = runner.step([StepEntry(i, [tails[i][k]], [0]) for i in range(live)])
+        errors += [gm.row_error(out[i].cpu(), want[i][len(prompts[i]) + k]) for i in range(live)]
+    gm.judge(errors, dtype)
+
+
 def test_long_decoding(backend, dtype, tmp_path_factory):
     """Hundreds of single-token steps after a short prompt: the state is carried, never
     rebuilt, and what the first tokens wrote still counts at the end (slow decays)."""
