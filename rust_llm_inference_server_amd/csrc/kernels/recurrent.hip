@@ -179,6 +179,23 @@ __device__ __forceinline__ float lanes_sum4(const float (&p)[4], int lane) {
   return xor32_sum(a);
 }
 
+// The same for two columns: lane l ends with the whole sum of column l % 2.
+__device__ __forceinline__ float lanes_sum2(const float (&p)[2], int lane) {
+  const bool odd = lane & 1;
+  float a = odd ? p[1] : p[0];
+  a += dpp_from<0xB1>(odd ? p[0] : p[1]);
+  a += dpp_from<0x4E>(a);    // two lanes on: the same column
+  a += dpp_from<0x124>(a);
+  a += dpp_from<0x128>(a);
+  a = xor16_sum(a);
+  return xor32_sum(a);
+}
+template <int NC>
+__device__ __forceinline__ float lanes_sum_cols(const float (&p)[NC], int lane) {
+  if constexpr (NC == 4) return lanes_sum4(p, lane);
+  else return lanes_sum2(p, lane);
+}
+
 // A wave walks kCols value channels of one (sequence, head): lane i holds S[i][j] of each (and
 // i + 64, ... for more than 64 key channels), so what a token brings per key channel is loaded
 // once for all of them and their sums over the wave interleave.  What does not depend on the
@@ -400,7 +417,7 @@ struct ScanTile {
   static constexpr int kKeys = KR * kWave;
 };
 
-template <int KR>
+template <int KR, int NC>
 __global__ __launch_bounds__(256) void delta_scan_tiled_kernel(
     float* __restrict__ out, long long ldo, const float* __restrict__ q, const float* __restrict__ k,
     const float* __restrict__ v, long long ldqkv, const float* __restrict__ b_raw,
@@ -408,12 +425,12 @@ __global__ __launch_bounds__(256) void delta_scan_tiled_kernel(
     const float* __restrict__ dt_bias, float* __restrict__ state, long long state_stride,
     const int* __restrict__ cu, const int* __restrict__ slots, int heads, int kv_heads, int dk,
     int dv) {
-  constexpr int TT = ScanTile<KR>::kTokens, DK = ScanTile<KR>::kKeys, CB = 4 * kCols;
+  constexpr int TT = ScanTile<KR>::kTokens, DK = ScanTile<KR>::kKeys, CB = 4 * NC, GROUP = kWave / NC;
   __shared__ float tk[TT][DK], tq[TT][DK], tv[TT][CB], tg[TT], tb[TT];
   const int lane = threadIdx.x % kWave;
   const int wave = threadIdx.x / kWave;
   const int jb = blockIdx.x * CB;                 // the workgroup's first column
-  const int j0 = jb + wave * kCols;
+  const int j0 = jb + wave * NC;
   const int head = blockIdx.y;
   const int s = blockIdx.z;
   const int kh = head / (heads / kv_heads);
@@ -427,9 +444,9 @@ __global__ __launch_bounds__(256) void delta_scan_tiled_kernel(
     idx[r] = i < dk ? i : dk - 1;
     live[r] = i < dk ? 1.f : 0.f;
   }
-  float S[kCols][KR];
+  float S[NC][KR];
 #pragma unroll
-  for (int c = 0; c < kCols; ++c) {
+  for (int c = 0; c < NC; ++c) {
     const int col = j0 + c < dv ? j0 + c : dv - 1;
 #pragma unroll
     for (int r = 0; r < KR; ++r) S[c][r] = base[(long long)col * dk + idx[r]] * live[r];
@@ -438,8 +455,8 @@ __global__ __launch_bounds__(256) void delta_scan_tiled_kernel(
   const float bias = dt_bias[head];
   // A tile's values wait in registers while the tile before is walked: every load of a tile is
   // asked for at once, and none of them is waited for before the walk in front of it is over.
-  constexpr int PER = TT * DK / 256, PERV = TT * CB / 256;
-  static_assert(TT * DK % 256 == 0 && TT * CB % 256 == 0 && TT <= 256, "tile sizes");
+  constexpr int PER = TT * DK / 256, PERV = (TT * CB + 255) / 256;
+  static_assert(TT * DK % 256 == 0 && TT <= 256, "tile sizes");
   float rk[PER], rq[PER], rv[PERV], rb = 0.f, rg = 0.f;
   auto ask = [&](int tile) {
     const int n = min(TT, t1 - tile);
@@ -454,7 +471,7 @@ __global__ __launch_bounds__(256) void delta_scan_tiled_kernel(
     }
 #pragma unroll
     for (int p = 0; p < PERV; ++p) {
-      const int e = threadIdx.x + p * 256, tt = e / CB, c = e % CB;
+      const int e = min(threadIdx.x + p * 256, TT * CB - 1), tt = e / CB, c = e % CB;
       const int col = jb + c < dv ? jb + c : dv - 1;
       rv[p] = v[(long long)(tile + (tt < n ? tt : n - 1)) * ldqkv + head * dv + col];
     }
@@ -476,7 +493,7 @@ __global__ __launch_bounds__(256) void delta_scan_tiled_kernel(
 #pragma unroll
     for (int p = 0; p < PERV; ++p) {
       const int e = threadIdx.x + p * 256;
-      tv[e / CB][e % CB] = rv[p];
+      if (e < TT * CB) tv[e / CB][e % CB] = rv[p];
     }
     if (threadIdx.x < TT) {
       tb[threadIdx.x] = sigmoidf_(rb);
@@ -487,19 +504,33 @@ __global__ __launch_bounds__(256) void delta_scan_tiled_kernel(
     // Lane l gathers the read-out of token (l / 4) of a group of sixteen for column l % 4 and
     // stores it when the group is through: one store a group, not four a token.
     float gathered = 0.f;
+    // a token's values are read from LDS while the token before it is worked on
+    float kx[KR], qx[KR], gx, bx, vx;
+    auto read = [&](int tt) {
+#pragma unroll
+      for (int r = 0; r < KR; ++r) {
+        kx[r] = tk[tt][lane + r * kWave];
+        qx[r] = tq[tt][lane + r * kWave];
+      }
+      gx = tg[tt];
+      bx = tb[tt];
+      vx = tv[tt][wave * NC + (lane & (NC - 1))];
+    };
+    read(0);
     for (int tt = 0; tt < n; ++tt) {
       float kc[KR], qc[KR], kq = 0.f;
 #pragma unroll
       for (int r = 0; r < KR; ++r) {
-        kc[r] = tk[tt][lane + r * kWave];
-        qc[r] = tq[tt][lane + r * kWave];
+        kc[r] = kx[r];
+        qc[r] = qx[r];
         kq += kc[r] * qc[r];
       }
-      const float g = tg[tt], beta = tb[tt];
-      const float v_own = tv[tt][wave * kCols + (lane & 3)];
-      float d1[kCols], d2[kCols];
+      const float g = gx, beta = bx;
+      const float v_own = vx;
+      read(tt + 1 < TT ? tt + 1 : tt);
+      float d1[NC], d2[NC];
 #pragma unroll
-      for (int c = 0; c < kCols; ++c) {
+      for (int c = 0; c < NC; ++c) {
         d1[c] = 0.f;
         d2[c] = 0.f;
 #pragma unroll
@@ -509,24 +540,29 @@ __global__ __launch_bounds__(256) void delta_scan_tiled_kernel(
         }
       }
       kq = lanes_sum(kq);
-      const float s1 = lanes_sum4(d1, lane), s2 = lanes_sum4(d2, lane);
+      const float s1 = lanes_sum_cols<NC>(d1, lane), s2 = lanes_sum_cols<NC>(d2, lane);
       const float u_own = beta * (v_own - g * s1);          // of column lane % 4
-      if ((lane >> 2) == (tt & 15)) gathered = g * s2 + kq * u_own;
-      const float u[kCols] = {dpp_from<0x00>(u_own), dpp_from<0x55>(u_own), dpp_from<0xAA>(u_own),
-                              dpp_from<0xFF>(u_own)};       // each column's, to every lane
+      if (lane / NC == tt % GROUP) gathered = g * s2 + kq * u_own;
+      float u[NC];                                          // each column's, to every lane
+      u[0] = dpp_from<0x00>(u_own);
+      u[1] = dpp_from<0x55>(u_own);
+      if constexpr (NC == 4) {
+        u[2] = dpp_from<0xAA>(u_own);
+        u[3] = dpp_from<0xFF>(u_own);
+      }
 #pragma unroll
-      for (int c = 0; c < kCols; ++c)
+      for (int c = 0; c < NC; ++c)
 #pragma unroll
         for (int r = 0; r < KR; ++r) S[c][r] = g * S[c][r] + kc[r] * u[c];
-      if ((tt & 15) == 15 || tt == n - 1) {
-        const int token = (tt & ~15) + (lane >> 2);
-        if (token <= tt && j0 + (lane & 3) < dv)
-          out[(long long)(tile + token) * ldo + head * dv + j0 + (lane & 3)] = gathered;
+      if (tt % GROUP == GROUP - 1 || tt == n - 1) {
+        const int token = tt / GROUP * GROUP + lane / NC;
+        if (token <= tt && j0 + (lane & (NC - 1)) < dv)
+          out[(long long)(tile + token) * ldo + head * dv + j0 + (lane & (NC - 1))] = gathered;
       }
     }
   }
 #pragma unroll
-  for (int c = 0; c < kCols; ++c)
+  for (int c = 0; c < NC; ++c)
     if (j0 + c < dv) {
 #pragma unroll
       for (int r = 0; r < KR; ++r)
@@ -534,24 +570,24 @@ __global__ __launch_bounds__(256) void delta_scan_tiled_kernel(
     }
 }
 
-template <int KR>
+template <int KR, int NC>
 __global__ __launch_bounds__(256) void decay_scan_tiled_kernel(
     float* __restrict__ out, const float* __restrict__ r_in, const float* __restrict__ k_in,
     const float* __restrict__ v_in, const float* __restrict__ z_in, long long ld,
     const float* __restrict__ w0, const float* __restrict__ bonus, float* __restrict__ state,
     long long state_stride, const int* __restrict__ cu, const int* __restrict__ slots, int heads,
     int d) {
-  constexpr int TT = ScanTile<KR>::kTokens / 2, DK = ScanTile<KR>::kKeys, CB = 4 * kCols;
+  constexpr int TT = ScanTile<KR>::kTokens / 2, DK = ScanTile<KR>::kKeys, CB = 4 * NC, GROUP = kWave / NC;
   __shared__ float tr[TT][DK], tk[TT][DK], tw[TT][DK], tv[TT][CB];
   const int lane = threadIdx.x % kWave;
   const int wave = threadIdx.x / kWave;
   const int jb = blockIdx.x * CB;
-  const int j0 = jb + wave * kCols;
+  const int j0 = jb + wave * NC;
   const int head = blockIdx.y;
   const int s = blockIdx.z;
   const int t0 = cu[s], t1 = cu[s + 1];
   float* base = state + (long long)slots[s] * state_stride + (long long)head * d * d;
-  float S[kCols][KR], u[KR];
+  float S[NC][KR], u[KR];
 #pragma unroll
   for (int r = 0; r < KR; ++r) {
     const int i = lane + r * kWave;
@@ -559,7 +595,7 @@ __global__ __launch_bounds__(256) void decay_scan_tiled_kernel(
     const float keep = i < d ? 1.f : 0.f;
     u[r] = bonus[head * d + ic];
 #pragma unroll
-    for (int c = 0; c < kCols; ++c) {
+    for (int c = 0; c < NC; ++c) {
       const int col = j0 + c < d ? j0 + c : d - 1;
       S[c][r] = base[(long long)col * d + ic] * keep;
     }
@@ -605,20 +641,36 @@ __global__ __launch_bounds__(256) void decay_scan_tiled_kernel(
     __syncthreads();
     ask(tile + TT < t1 ? tile + TT : tile);
     float gathered = 0.f;                          // as in the kernel above
-    for (int tt = 0; tt < n; ++tt) {
-      float rc[KR], kc[KR], wc[KR], ruk = 0.f;
+    float rx[KR], kx[KR], wx[KR], vx, vcx[NC];
+    auto read = [&](int tt) {
 #pragma unroll
       for (int r = 0; r < KR; ++r) {
-        rc[r] = tr[tt][lane + r * kWave];
-        kc[r] = tk[tt][lane + r * kWave];
-        wc[r] = tw[tt][lane + r * kWave];
+        rx[r] = tr[tt][lane + r * kWave];
+        kx[r] = tk[tt][lane + r * kWave];
+        wx[r] = tw[tt][lane + r * kWave];
+      }
+      vx = tv[tt][wave * NC + (lane & (NC - 1))];
+#pragma unroll
+      for (int c = 0; c < NC; ++c) vcx[c] = tv[tt][wave * NC + c];
+    };
+    read(0);
+    for (int tt = 0; tt < n; ++tt) {
+      float rc[KR], kc[KR], wc[KR], vcs[NC], ruk = 0.f;
+#pragma unroll
+      for (int r = 0; r < KR; ++r) {
+        rc[r] = rx[r];
+        kc[r] = kx[r];
+        wc[r] = wx[r];
         ruk += rc[r] * u[r] * kc[r];
       }
-      const float v_own = tv[tt][wave * kCols + (lane & 3)];
-      float o[kCols];
+      const float v_own = vx;
 #pragma unroll
-      for (int c = 0; c < kCols; ++c) {
-        const float vc = tv[tt][wave * kCols + c];
+      for (int c = 0; c < NC; ++c) vcs[c] = vcx[c];
+      read(tt + 1 < TT ? tt + 1 : tt);
+      float o[NC];
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        const float vc = vcs[c];
         o[c] = 0.f;
 #pragma unroll
         for (int r = 0; r < KR; ++r) {
@@ -627,17 +679,17 @@ __global__ __launch_bounds__(256) void decay_scan_tiled_kernel(
         }
       }
       ruk = lanes_sum(ruk);
-      const float total = lanes_sum4(o, lane);
-      if ((lane >> 2) == (tt & 15)) gathered = total + ruk * v_own;
-      if ((tt & 15) == 15 || tt == n - 1) {
-        const int token = (tt & ~15) + (lane >> 2);
-        if (token <= tt && j0 + (lane & 3) < d)
-          out[(long long)(tile + token) * ld + head * d + j0 + (lane & 3)] = gathered;
+      const float total = lanes_sum_cols<NC>(o, lane);
+      if (lane / NC == tt % GROUP) gathered = total + ruk * v_own;
+      if (tt % GROUP == GROUP - 1 || tt == n - 1) {
+        const int token = tt / GROUP * GROUP + lane / NC;
+        if (token <= tt && j0 + (lane & (NC - 1)) < d)
+          out[(long long)(tile + token) * ld + head * d + j0 + (lane & (NC - 1))] = gathered;
       }
     }
   }
 #pragma unroll
-  for (int c = 0; c < kCols; ++c)
+  for (int c = 0; c < NC; ++c)
     if (j0 + c < d) {
 #pragma unroll
       for (int r = 0; r < KR; ++r)
@@ -668,6 +720,17 @@ __global__ __launch_bounds__(kWave) void head_norm_gate_kernel(
 }  // namespace
 
 // ============================================================================ entry points
+static int scan_compute_units() {
+  static int units = 0;
+  if (units == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    units = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+                ? prop.multiProcessorCount : 256;
+  }
+  return units;
+}
+
 RLIS_API int rlis_shift_mix(void* out, const void* x, int dtype, const float* mu,
                             const float* state, long long state_stride, const int* seq_of_token,
                             const int* cu, const int* slots, int T, int W, int mixes,
@@ -754,16 +817,24 @@ RLIS_API int rlis_delta_scan(float* out, long long ldo, const float* q, const fl
   delta_scan_kernel<KR><<<grid, 256, 0, stream>>>(out, ldo, q, k, v, ldqkv, b_raw, a_raw, ldba, \
                                                   a_log, dt_bias, state, state_stride, cu,    \
                                                   slots, heads, kv_heads, dk, dv)
+  // Few workgroups (a single prompt): two value channels a wave instead of four, twice the waves.
+  // (tiled 2 / 3: four / two channels a wave whatever the grid, for tests)
+  const bool narrow = tiled == 3 || (tiled == 1 && (long long)grid.x * heads * num_seqs < 2 * scan_compute_units());
+  const dim3 grid2(ceil_div(dv, 4 * 2), heads, num_seqs);
 #define LAUNCH_TILED(KR)                                                                      \
-  delta_scan_tiled_kernel<KR><<<grid, 256, 0, stream>>>(out, ldo, q, k, v, ldqkv, b_raw, a_raw, \
-                                                        ldba, a_log, dt_bias, state,          \
-                                                        state_stride, cu, slots, heads,       \
-                                                        kv_heads, dk, dv)
+  if (narrow)                                                                                 \
+    delta_scan_tiled_kernel<KR, 2><<<grid2, 256, 0, stream>>>(                                \
+        out, ldo, q, k, v, ldqkv, b_raw, a_raw, ldba, a_log, dt_bias, state, state_stride, cu, \
+        slots, heads, kv_heads, dk, dv);                                                      \
+  else                                                                                        \
+    delta_scan_tiled_kernel<KR, kCols><<<grid, 256, 0, stream>>>(                             \
+        out, ldo, q, k, v, ldqkv, b_raw, a_raw, ldba, a_log, dt_bias, state, state_stride, cu, \
+        slots, heads, kv_heads, dk, dv)
   // `tiled`: some sequence of the step brings many tokens (the caller knows from the host)
   if (tiled) {
-    if (dk <= 64) LAUNCH_TILED(1);
-    else if (dk <= 128) LAUNCH_TILED(2);
-    else LAUNCH_TILED(4);
+    if (dk <= 64) { LAUNCH_TILED(1); }
+    else if (dk <= 128) { LAUNCH_TILED(2); }
+    else { LAUNCH_TILED(4); }
   } else if (dk <= 64) LAUNCH(1);
   else if (dk <= 128) LAUNCH(2);
   else LAUNCH(4);
@@ -788,13 +859,21 @@ RLIS_API int rlis_decay_scan(float* out, const float* r, const float* k, const f
 #define LAUNCH(KR)                                                                           \
   decay_scan_kernel<KR><<<grid, 256, 0, stream>>>(out, r, k, v, z, ld, w0, bonus, state,     \
                                                   state_stride, cu, slots, heads, d)
+  const bool narrow = tiled == 3 || (tiled == 1 && (long long)grid.x * heads * num_seqs < 2 * scan_compute_units());
+  const dim3 grid2(ceil_div(d, 4 * 2), heads, num_seqs);
 #define LAUNCH_TILED(KR)                                                                     \
-  decay_scan_tiled_kernel<KR><<<grid, 256, 0, stream>>>(out, r, k, v, z, ld, w0, bonus, state, \
-                                                        state_stride, cu, slots, heads, d)
+  if (narrow)                                                                                \
+    decay_scan_tiled_kernel<KR, 2><<<grid2, 256, 0, stream>>>(out, r, k, v, z, ld, w0, bonus, \
+                                                              state, state_stride, cu, slots, \
+                                                              heads, d);                     \
+  else                                                                                       \
+    decay_scan_tiled_kernel<KR, kCols><<<grid, 256, 0, stream>>>(out, r, k, v, z, ld, w0,     \
+                                                                 bonus, state, state_stride, \
+                                                                 cu, slots, heads, d)
   if (tiled) {
-    if (d <= 64) LAUNCH_TILED(1);
-    else if (d <= 128) LAUNCH_TILED(2);
-    else LAUNCH_TILED(4);
+    if (d <= 64) { LAUNCH_TILED(1); }
+    else if (d <= 128) { LAUNCH_TILED(2); }
+    else { LAUNCH_TILED(4); }
   } else if (d <= 64) LAUNCH(1);
   else if (d <= 128) LAUNCH(2);
   else LAUNCH(4);

@@ -64,6 +64,15 @@ def _long_runs(T: int, num_seqs: int) -> bool:
     return T >= TILED_SCAN_MIN_MEAN_TOKENS * max(1, num_seqs)
 
 
+def _scan_form(tiled, T: int, num_seqs: int) -> int:
+    """The kernels' form argument: 0 the streaming kernel, 1 the tiled one (two value channels a
+    wave where the grid is small, else four), 2 / 3 the tiled one with four / two channels a
+    wave (``"wide"`` / ``"narrow"``, for tests)."""
+    if tiled is None:
+        tiled = _long_runs(T, num_seqs)
+    return {False: 0, True: 1, "wide": 2, "narrow": 3}[tiled]
+
+
 def shift_mix(x: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, seq_of_token: torch.Tensor,
               cu: torch.Tensor, slots: torch.Tensor, num_seqs: int) -> torch.Tensor:
     """``out[m] = x + (prev - x) * mu[m]`` for every row of ``x (T, W)``, ``prev`` being the row
@@ -125,7 +134,7 @@ def delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, b_raw: torch.T
                a_raw: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor,
                state: torch.Tensor, cu: torch.Tensor, slots: torch.Tensor, num_seqs: int,
                heads: int, kv_heads: int, dk: int, dv: int,
-               tiled: Optional[bool] = None) -> torch.Tensor:
+               tiled=None) -> torch.Tensor:
     """The gated delta rule over every sequence's tokens of the step.  ``q``, ``k``
     ``(T, kv_heads * dk)`` and ``v (T, heads * dv)`` are float32 column ranges of one matrix
     (one row stride), ``b_raw``, ``a_raw`` ``(T, heads)`` of another; per token and head
@@ -153,14 +162,14 @@ def delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, b_raw: torch.T
              _vec(a_log, heads, "delta_scan A_log"), _vec(dt_bias, heads, "delta_scan dt_bias"),
              state.data_ptr(), stride, _meta(cu, num_seqs + 1, "cu"),
              _meta(slots, num_seqs, "slots"), num_seqs, heads, kv_heads, dk, dv,
-             int(_long_runs(T, num_seqs) if tiled is None else bool(tiled)), lib.stream_ptr())
+             _scan_form(tiled, T, num_seqs), lib.stream_ptr())
     return out
 
 
 def decay_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch.Tensor,
                w0: torch.Tensor, bonus: torch.Tensor, state: torch.Tensor, cu: torch.Tensor,
                slots: torch.Tensor, num_seqs: int, heads: int, d: int,
-               tiled: Optional[bool] = None) -> torch.Tensor:
+               tiled=None) -> torch.Tensor:
     """A matrix state per head with a decay per key channel and a bonus for the current token:
     per token ``o = (S + diag(bonus) k v^T)^T r; S <- diag(w) S + k v^T`` with
     ``w = exp(-exp(z + w0))``.  ``r``, ``k``, ``v``, ``z`` are contiguous float32
@@ -177,7 +186,7 @@ def decay_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch.Tenso
              z.data_ptr(), heads * d, _vec(w0, heads * d, "decay_scan w0"),
              _vec(bonus.reshape(-1), heads * d, "decay_scan bonus"), state.data_ptr(), stride,
              _meta(cu, num_seqs + 1, "cu"), _meta(slots, num_seqs, "slots"), num_seqs, heads, d,
-             int(_long_runs(T, num_seqs) if tiled is None else bool(tiled)), lib.stream_ptr())
+             _scan_form(tiled, T, num_seqs), lib.stream_ptr())
     return out
 
 

@@ -42,11 +42,12 @@ def _cut(x, lengths_by_step, step, seq):
     return slice(start, start + lengths_by_step[step][seq])
 
 
-@pytest.mark.parametrize("tiled", [False, True, None])
+@pytest.mark.parametrize("tiled", [False, "wide", "narrow", None])
 @pytest.mark.parametrize("heads, d", [(3, 16), (2, 96), (1, 160), (2, 50)])
 def test_decayed_state_scan(heads, d, tiled):
-    """``tiled``: the kernel that stages tiles of tokens through LDS, the one that asks for a
-    token's vectors one token ahead, or whichever the step's shape chooses."""
+    """``tiled``: the kernel that asks for a token's vectors one token ahead, the one that stages
+    tiles of tokens through LDS with four or with two value channels a wave, or whichever the
+    step's shape chooses."""
     ops = _ops()
     g = torch.Generator().manual_seed(heads * 100 + d)
     totals = [sum(s[i] for s in STEPS) for i in range(3)]
@@ -79,7 +80,7 @@ def test_decayed_state_scan(heads, d, tiled):
     assert float(buf[1].min()) == 7.5 and float(buf[:, :8].min()) == 7.5     # nothing else moved
 
 
-@pytest.mark.parametrize("tiled", [False, True, None])
+@pytest.mark.parametrize("tiled", [False, "wide", "narrow", None])
 @pytest.mark.parametrize("heads, groups, dk, dv", [(4, 2, 16, 24), (2, 1, 96, 6), (1, 1, 200, 33),
                                                    (6, 3, 64, 64)])
 def test_gated_delta_scan(heads, groups, dk, dv, tiled):
