@@ -311,6 +311,29 @@ def test_greedy_generation_through_the_engine(backend, dtype, tmp_path_factory):
     engine.runner.cache.check_invariants()
 
 
+def test_preempted_requests_recompute_their_state(backend, tmp_path_factory):
+    """So few pages that running requests are parked and later recomputed from their first
+    token: their state slots are cleared and rebuilt, and the tokens are those of a roomy run."""
+    from rust_llm_inference_server_amd.engine import Engine, load_model
+    folder, cfg, stored = model_case("b", "float32", tmp_path_factory)
+    model = load_model(folder, "float32", 128, backend)
+    prompts = gm.prompts(cfg["vocab"], [9] * 6, seed=25)
+    sp = SamplingParams.greedy(20)
+    runs = []
+    for pages in (64, 12):
+        engine = Engine(model, EngineConfig(max_num_seqs=6, max_batched_tokens=64, num_pages=pages,
+                                            block_size=8, max_seq_len=128, watermark_pages=0))
+        runs.append([o.token_ids for o in engine.generate(prompts, sp)])
+        assert (engine.stats().preemptions > 0) == (pages == 12)
+        assert engine.runner.cache.num_free_pages() == pages
+        engine.runner.cache.check_invariants()
+    for roomy, tight, p in zip(runs[0], runs[1], prompts):
+        if roomy != tight:                      # only at a near-tie of the plain logits
+            at = next(i for i, (a, b) in enumerate(zip(roomy, tight)) if a != b)
+            last = plain.forward(cfg, stored, list(p) + roomy[:at])[-1]
+            assert abs(float(last[roomy[at]] - last[tight[at]])) < 1e-3
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
 def test_the_replay_program_runs_the_model(dtype_name, tmp_path_factory, tmp_path):
