@@ -631,7 +631,7 @@ __global__ __launch_bounds__(256) void decay_scan_tiled_kernel(
       const int e = threadIdx.x + p * 256;
       tr[e / DK][e % DK] = rr[p];
       tk[e / DK][e % DK] = rk[p];
-      tw[e / DK][e % DK] = expf(-expf(rz[p]));
+      tw[e / DK][e % DK] = e / DK < n ? expf(-expf(rz[p])) : 1.f;   // no decay past the end
     }
 #pragma unroll
     for (int p = 0; p < PERV; ++p) {
@@ -640,50 +640,58 @@ __global__ __launch_bounds__(256) void decay_scan_tiled_kernel(
     }
     __syncthreads();
     ask(tile + TT < t1 ? tile + TT : tile);
+    // Four tokens at a time: their read-outs are sums over the state before each of them, and
+    // nothing in the state waits for a sum, so the four tokens' sums over the wave are formed
+    // side by side (independent chains fill the slots that one chain leaves empty), and
+    // four tokens' bonus terms r.u.k in one four-column sum.  Tokens past the end carry r = k = 0
+    // and w = 1: they leave the state as it is and are not stored.
     float gathered = 0.f;                          // as in the kernel above
-    float rx[KR], kx[KR], wx[KR], vx, vcx[NC];
-    auto read = [&](int tt) {
+    constexpr int U = 4;                           // eight at a time were no faster
+    static_assert(TT % U == 0 && GROUP % U == 0 && U % 4 == 0, "token groups");
+    for (int tb = 0; tb < n; tb += U) {
+      float o[U][NC], ruk[U], v_own[U];
 #pragma unroll
-      for (int r = 0; r < KR; ++r) {
-        rx[r] = tr[tt][lane + r * kWave];
-        kx[r] = tk[tt][lane + r * kWave];
-        wx[r] = tw[tt][lane + r * kWave];
-      }
-      vx = tv[tt][wave * NC + (lane & (NC - 1))];
-#pragma unroll
-      for (int c = 0; c < NC; ++c) vcx[c] = tv[tt][wave * NC + c];
-    };
-    read(0);
-    for (int tt = 0; tt < n; ++tt) {
-      float rc[KR], kc[KR], wc[KR], vcs[NC], ruk = 0.f;
-#pragma unroll
-      for (int r = 0; r < KR; ++r) {
-        rc[r] = rx[r];
-        kc[r] = kx[r];
-        wc[r] = wx[r];
-        ruk += rc[r] * u[r] * kc[r];
-      }
-      const float v_own = vx;
-#pragma unroll
-      for (int c = 0; c < NC; ++c) vcs[c] = vcx[c];
-      read(tt + 1 < TT ? tt + 1 : tt);
-      float o[NC];
-#pragma unroll
-      for (int c = 0; c < NC; ++c) {
-        const float vc = vcs[c];
-        o[c] = 0.f;
+      for (int uu = 0; uu < U; ++uu) {
+        const int tt = tb + uu;
+        float rc[KR], kc[KR], wc[KR];
+        ruk[uu] = 0.f;
 #pragma unroll
         for (int r = 0; r < KR; ++r) {
-          o[c] += rc[r] * S[c][r];
-          S[c][r] = wc[r] * S[c][r] + kc[r] * vc;
+          rc[r] = tr[tt][lane + r * kWave];
+          kc[r] = tk[tt][lane + r * kWave];
+          wc[r] = tw[tt][lane + r * kWave];
+          ruk[uu] += rc[r] * u[r] * kc[r];
+        }
+        v_own[uu] = tv[tt][wave * NC + (lane & (NC - 1))];
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+          const float vc = tv[tt][wave * NC + c];
+          o[uu][c] = 0.f;
+#pragma unroll
+          for (int r = 0; r < KR; ++r) {
+            o[uu][c] += rc[r] * S[c][r];
+            S[c][r] = wc[r] * S[c][r] + kc[r] * vc;
+          }
         }
       }
-      ruk = lanes_sum(ruk);
-      const float total = lanes_sum_cols<NC>(o, lane);
-      if (lane / NC == tt % GROUP) gathered = total + ruk * v_own;
-      if (tt % GROUP == GROUP - 1 || tt == n - 1) {
-        const int token = tt / GROUP * GROUP + lane / NC;
-        if (token <= tt && j0 + (lane & (NC - 1)) < d)
+      float ruk_all[U];                                      // each token's, to every lane
+#pragma unroll
+      for (int q4 = 0; q4 < U; q4 += 4) {
+        const float four[4] = {ruk[q4], ruk[q4 + 1], ruk[q4 + 2], ruk[q4 + 3]};
+        const float mine = lanes_sum4(four, lane);           // of token q4 + lane % 4
+        ruk_all[q4] = dpp_from<0x00>(mine);
+        ruk_all[q4 + 1] = dpp_from<0x55>(mine);
+        ruk_all[q4 + 2] = dpp_from<0xAA>(mine);
+        ruk_all[q4 + 3] = dpp_from<0xFF>(mine);
+      }
+#pragma unroll
+      for (int uu = 0; uu < U; ++uu) {
+        const float total = lanes_sum_cols<NC>(o[uu], lane);
+        if (lane / NC == (tb + uu) % GROUP) gathered = total + ruk_all[uu] * v_own[uu];
+      }
+      if ((tb + U) % GROUP == 0 || tb + U >= n) {
+        const int token = tb / GROUP * GROUP + lane / NC;
+        if (token < n && token < tb + U && j0 + (lane & (NC - 1)) < d)
           out[(long long)(tile + token) * ld + head * d + j0 + (lane & (NC - 1))] = gathered;
       }
     }
