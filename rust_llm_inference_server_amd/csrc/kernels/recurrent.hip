@@ -417,6 +417,11 @@ struct ScanTile {
   static constexpr int kKeys = KR * kWave;
 };
 
+#ifndef RLIS_DELTA_GROUP
+#define RLIS_DELTA_GROUP 2
+#endif
+constexpr int kDeltaGroup = RLIS_DELTA_GROUP;   // tokens whose sums run side by side
+
 template <int KR, int NC>
 __global__ __launch_bounds__(256) void delta_scan_tiled_kernel(
     float* __restrict__ out, long long ldo, const float* __restrict__ q, const float* __restrict__ k,
@@ -426,7 +431,9 @@ __global__ __launch_bounds__(256) void delta_scan_tiled_kernel(
     const int* __restrict__ cu, const int* __restrict__ slots, int heads, int kv_heads, int dk,
     int dv) {
   constexpr int TT = ScanTile<KR>::kTokens, DK = ScanTile<KR>::kKeys, CB = 4 * NC, GROUP = kWave / NC;
+  constexpr int U = kDeltaGroup;
   __shared__ float tk[TT][DK], tq[TT][DK], tv[TT][CB], tg[TT], tb[TT];
+  __shared__ __attribute__((aligned(16))) float tp[TT / U][U * U];
   const int lane = threadIdx.x % kWave;
   const int wave = threadIdx.x / kWave;
   const int jb = blockIdx.x * CB;                 // the workgroup's first column
@@ -495,68 +502,131 @@ __global__ __launch_bounds__(256) void delta_scan_tiled_kernel(
       const int e = threadIdx.x + p * 256;
       if (e < TT * CB) tv[e / CB][e % CB] = rv[p];
     }
-    if (threadIdx.x < TT) {
-      tb[threadIdx.x] = sigmoidf_(rb);
-      tg[threadIdx.x] = expf(neg_a * softplusf_(rg + bias));
+    if (threadIdx.x < TT) {                        // past the end: no step, no decay
+      tb[threadIdx.x] = threadIdx.x < n ? sigmoidf_(rb) : 0.f;
+      tg[threadIdx.x] = threadIdx.x < n ? expf(neg_a * softplusf_(rg + bias)) : 1.f;
     }
     __syncthreads();
     ask(tile + TT < t1 ? tile + TT : tile);
-    // Lane l gathers the read-out of token (l / 4) of a group of sixteen for column l % 4 and
-    // stores it when the group is through: one store a group, not four a token.
+    // Lane l gathers the read-out of token (l / NC) of a group for column l % NC and stores it
+    // when the group is through: one store a group, not NC a token.
     float gathered = 0.f;
-    // a token's values are read from LDS while the token before it is worked on
-    float kx[KR], qx[KR], gx, bx, vx;
-    auto read = [&](int tt) {
+    // U tokens at a time.  With S the state in front of the group, G(t) the product of the
+    // decays up to token t and G(t, s) that of tokens s + 1 .. t:
+    //   u_t = beta_t (v_t - G(t) S^T k_t - sum_{s<t} G(t, s) (k_s . k_t) u_s)
+    //   o_t = G(t) S^T q_t + sum_{s<=t} G(t, s) (k_s . q_t) u_s
+    //   S  <- G(U-1) S + sum_s G(U-1, s) k_s u_s^T
+    // so every sum over the wave is over the state in front of the group or over the tokens'
+    // own vectors: all of a group's sums run side by side, and the state waits for them once a
+    // group, not once a token.  Tokens past the end carry k = q = 0, beta = 0, g = 1.
+    static_assert(TT % U == 0 && GROUP % U == 0 && (TT * U) % 16 == 0, "token groups");
+    // The tokens' own products, once a tile for all its groups and all four waves: entry (a, b)
+    // of a group is k_b . q_a for b <= a and k_a . k_b for b > a; a wave sums four entries at
+    // a time and lanes 0 to 3 put them down.
+    {
+      float* flat = &tp[0][0];
+      for (int f = wave * 4; f < TT * U; f += 16) {
+        float four[4];
 #pragma unroll
-      for (int r = 0; r < KR; ++r) {
-        kx[r] = tk[tt][lane + r * kWave];
-        qx[r] = tq[tt][lane + r * kWave];
+        for (int m = 0; m < 4; ++m) {
+          const int e = f + m, first = e / (U * U) * U, a2 = e % (U * U) / U, b2 = e % U;
+          const float* other = b2 <= a2 ? tq[first + a2] : tk[first + a2];
+          float pp = 0.f;
+#pragma unroll
+          for (int r = 0; r < KR; ++r) pp += tk[first + b2][lane + r * kWave] * other[lane + r * kWave];
+          four[m] = pp;
+        }
+        const float mine = lanes_sum4(four, lane);           // of entry f + lane % 4
+        if (lane < 4) flat[f + lane] = mine;
       }
-      gx = tg[tt];
-      bx = tb[tt];
-      vx = tv[tt][wave * NC + (lane & (NC - 1))];
-    };
-    read(0);
-    for (int tt = 0; tt < n; ++tt) {
-      float kc[KR], qc[KR], kq = 0.f;
+    }
+    __syncthreads();
+    for (int tb0 = 0; tb0 < n; tb0 += U) {
+      float kc[U][KR], qc[U][KR], g[U], beta[U], v_own[U];
 #pragma unroll
-      for (int r = 0; r < KR; ++r) {
-        kc[r] = kx[r];
-        qc[r] = qx[r];
-        kq += kc[r] * qc[r];
-      }
-      const float g = gx, beta = bx;
-      const float v_own = vx;
-      read(tt + 1 < TT ? tt + 1 : tt);
-      float d1[NC], d2[NC];
-#pragma unroll
-      for (int c = 0; c < NC; ++c) {
-        d1[c] = 0.f;
-        d2[c] = 0.f;
+      for (int t = 0; t < U; ++t) {
 #pragma unroll
         for (int r = 0; r < KR; ++r) {
-          d1[c] += S[c][r] * kc[r];
-          d2[c] += S[c][r] * qc[r];
+          kc[t][r] = tk[tb0 + t][lane + r * kWave];
+          qc[t][r] = tq[tb0 + t][lane + r * kWave];
+        }
+        g[t] = tg[tb0 + t];
+        beta[t] = tb[tb0 + t];
+        v_own[t] = tv[tb0 + t][wave * NC + (lane & (NC - 1))];
+      }
+      float pair[U * U];
+#pragma unroll
+      for (int f = 0; f < U * U; ++f) pair[f] = tp[tb0 / U][f];
+      // the sums over the state in front of the group, for this lane's column
+      float s1[U], s2[U];
+#pragma unroll
+      for (int t = 0; t < U; ++t) {
+        float d1[NC], d2[NC];
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+          d1[c] = 0.f;
+          d2[c] = 0.f;
+#pragma unroll
+          for (int r = 0; r < KR; ++r) {
+            d1[c] += S[c][r] * kc[t][r];
+            d2[c] += S[c][r] * qc[t][r];
+          }
+        }
+        if constexpr (NC == 2) {       // both sums of both columns in one four-column sum
+          const float four[4] = {d1[0], d1[1], d2[0], d2[1]};
+          const float mine = lanes_sum4(four, lane);
+          s1[t] = dpp_from<0x44>(mine);                      // quad_perm [0, 1, 0, 1]
+          s2[t] = dpp_from<0xEE>(mine);                      // quad_perm [2, 3, 2, 3]
+        } else {
+          s1[t] = lanes_sum_cols<NC>(d1, lane);
+          s2[t] = lanes_sum_cols<NC>(d2, lane);
         }
       }
-      kq = lanes_sum(kq);
-      const float s1 = lanes_sum_cols<NC>(d1, lane), s2 = lanes_sum_cols<NC>(d2, lane);
-      const float u_own = beta * (v_own - g * s1);          // of column lane % 4
-      if (lane / NC == tt % GROUP) gathered = g * s2 + kq * u_own;
-      float u[NC];                                          // each column's, to every lane
-      u[0] = dpp_from<0x00>(u_own);
-      u[1] = dpp_from<0x55>(u_own);
-      if constexpr (NC == 4) {
-        u[2] = dpp_from<0xAA>(u_own);
-        u[3] = dpp_from<0xFF>(u_own);
+      // the group's recurrence in scalars, for the column lane % NC
+      float gam[U][U], upto[U], u_own[U];
+#pragma unroll
+      for (int t = 0; t < U; ++t) {
+        upto[t] = t ? upto[t - 1] * g[t] : g[t];
+        gam[t][t] = 1.f;
+#pragma unroll
+        for (int s0 = 0; s0 < t; ++s0) gam[t][s0] = gam[t - 1][s0] * g[t];
+      }
+#pragma unroll
+      for (int t = 0; t < U; ++t) {
+        float inner = upto[t] * s1[t], o = upto[t] * s2[t];
+#pragma unroll
+        for (int s0 = 0; s0 < t; ++s0) {
+          inner += gam[t][s0] * pair[s0 * U + t] * u_own[s0];
+          o += gam[t][s0] * pair[t * U + s0] * u_own[s0];
+        }
+        u_own[t] = beta[t] * (v_own[t] - inner);
+        o += pair[t * U + t] * u_own[t];
+        if (lane / NC == (tb0 + t) % GROUP) gathered = o;
+      }
+      // each column's steps to every lane, and the state behind the group
+      float coef[U][NC];
+#pragma unroll
+      for (int t = 0; t < U; ++t) {
+        const float scaled = gam[U - 1][t] * u_own[t];
+        coef[t][0] = dpp_from<0x00>(scaled);
+        coef[t][1] = dpp_from<0x55>(scaled);
+        if constexpr (NC == 4) {
+          coef[t][2] = dpp_from<0xAA>(scaled);
+          coef[t][3] = dpp_from<0xFF>(scaled);
+        }
       }
 #pragma unroll
       for (int c = 0; c < NC; ++c)
 #pragma unroll
-        for (int r = 0; r < KR; ++r) S[c][r] = g * S[c][r] + kc[r] * u[c];
-      if (tt % GROUP == GROUP - 1 || tt == n - 1) {
-        const int token = tt / GROUP * GROUP + lane / NC;
-        if (token <= tt && j0 + (lane & (NC - 1)) < dv)
+        for (int r = 0; r < KR; ++r) {
+          float acc = upto[U - 1] * S[c][r];
+#pragma unroll
+          for (int t = 0; t < U; ++t) acc += kc[t][r] * coef[t][c];
+          S[c][r] = acc;
+        }
+      if ((tb0 + U) % GROUP == 0 || tb0 + U >= n) {
+        const int token = tb0 / GROUP * GROUP + lane / NC;
+        if (token < n && token < tb0 + U && j0 + (lane & (NC - 1)) < dv)
           out[(long long)(tile + token) * ldo + head * dv + j0 + (lane & (NC - 1))] = gathered;
       }
     }
