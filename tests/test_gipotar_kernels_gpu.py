@@ -31,8 +31,9 @@ def _state(num_slots, used, extra=24):
     return buf, buf[:, 8:8 + used]
 
 
-# tokens per sequence, step by step (a run longer than a tile of the tiled scans among them)
-STEPS = [[5, 1, 9], [1, 1, 2], [3, 1, 1], [17, 2, 1], [2, 70, 33]]
+# tokens per sequence, step by step (runs longer than a tile of the tiled scans among them, and
+# runs that end one token short of a tile, at its end, and inside a group of tokens behind it)
+STEPS = [[5, 1, 9], [1, 1, 2], [3, 1, 1], [17, 2, 1], [2, 70, 33], [31, 32, 34], [15, 16, 7]]
 SLOTS = [3, 0, 2]
 
 
