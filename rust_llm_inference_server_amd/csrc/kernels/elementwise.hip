@@ -944,3 +944,92 @@ RLIS_API int rlis_fill_normal_device(void* out, int out_dtype, long long n, unsi
   RLIS_LAUNCH_CHECK("fill_normal");
   return 0;
 }
+
+// ------------------------------------------------------------------ layer norm
+// out = (x - mean) / sqrt(var + eps) * weight + bias over a row of x = resid + scale * delta
+// (delta optional; a stack of float32 partial sums is added in order, and with round_parts
+// rounded to bfloat16 first), var the mean of the squared deviations from the mean.  The
+// sum is stored back into the residual when write_resid is set; with `rows` only those rows
+// are made and the residual stays.  Sum, statistics and both multiplies are float32; the row
+// waits in LDS between the passes (one read of the operands).
+template <typename TD, typename TW, typename TO>
+__global__ __launch_bounds__(256) void add_layernorm_kernel(
+    float* __restrict__ resid, const TD* __restrict__ delta, const TW* __restrict__ weight,
+    const TW* __restrict__ bias, TO* __restrict__ out, const int* __restrict__ rows, int H,
+    float eps, int write_resid, int parts, long long part_stride, int round_parts,
+    float delta_scale) {
+  extern __shared__ float row_s[];
+  __shared__ float red[4];
+  const int r = blockIdx.x;
+  const long long src = rows ? rows[r] : r;
+  float* xr = resid + src * H;
+  float sum = 0.f;
+  for (int j = threadIdx.x; j < H; j += 256) {
+    float v = xr[j];
+    if (delta) v += delta_scale * delta_sum(delta + src * H + j, parts, part_stride, round_parts);
+    row_s[j] = v;
+    if (write_resid) xr[j] = v;
+    sum += v;
+  }
+  const float mean = block_sum<256>(sum, red) / (float)H;
+  float sq = 0.f;
+  for (int j = threadIdx.x; j < H; j += 256) {
+    const float d = row_s[j] - mean;
+    sq += d * d;
+  }
+  const float mult = 1.0f / sqrtf(block_sum<256>(sq, red) / (float)H + eps);
+  for (int j = threadIdx.x; j < H; j += 256)
+    st(out + (long long)r * H + j, (row_s[j] - mean) * mult * widen(weight[j]) + widen(bias[j]));
+}
+
+RLIS_API int rlis_add_layernorm(float* resid, const void* delta, int delta_dtype,
+                                const void* weight, const void* bias, int weight_dtype, void* out,
+                                int out_dtype, const int* rows, int R, int H, float eps,
+                                int write_resid, int parts, long long part_stride,
+                                int round_parts, float delta_scale, hipStream_t stream) {
+  RLIS_REQUIRE(R >= 0 && H > 0 && H <= 16000, "add_layernorm: bad sizes R=%d H=%d", R, H);
+  RLIS_REQUIRE(parts >= 1, "add_layernorm: parts=%d", parts);
+  RLIS_REQUIRE(!(rows && write_resid && delta),
+               "add_layernorm: writing the residual back needs all rows, not a selection");
+  if (R == 0) return 0;
+  const int key = (delta ? delta_dtype : RLIS_F32) * 4 + weight_dtype * 2 + out_dtype;
+#define CASE(k, TD, TW, TO)                                                                  \
+  case k:                                                                                    \
+    add_layernorm_kernel<TD, TW, TO><<<R, 256, (size_t)H * 4, stream>>>(                     \
+        resid, (const TD*)delta, (const TW*)weight, (const TW*)bias, (TO*)out, rows, H, eps, \
+        write_resid && delta, parts, part_stride, round_parts, delta_scale);                 \
+    break;
+  switch (key) {
+    CASE(0, float, float, float)
+    CASE(1, float, float, bf16_t)
+    CASE(2, float, bf16_t, float)
+    CASE(3, float, bf16_t, bf16_t)
+    CASE(4, bf16_t, float, float)
+    CASE(5, bf16_t, float, bf16_t)
+    CASE(6, bf16_t, bf16_t, float)
+    CASE(7, bf16_t, bf16_t, bf16_t)
+    default:
+      RLIS_REQUIRE(false, "add_layernorm: unknown dtypes");
+  }
+#undef CASE
+  RLIS_LAUNCH_CHECK("add_layernorm");
+  return 0;
+}
+
+// x <- x * factor in place (float32 product, one rounding).
+template <typename TX>
+__global__ void scale_kernel(TX* __restrict__ x, long long n, float factor) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) st(x + i, ld(x + i) * factor);
+}
+
+RLIS_API int rlis_scale(void* x, int dtype, long long n, float factor, hipStream_t stream) {
+  RLIS_REQUIRE(n >= 0, "scale: bad size");
+  if (n == 0) return 0;
+  const unsigned blocks = (unsigned)ceil_div_ll(n, 256);
+  if (dtype == RLIS_F32) scale_kernel<float><<<blocks, 256, 0, stream>>>((float*)x, n, factor);
+  else if (dtype == RLIS_BF16) scale_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)x, n, factor);
+  else RLIS_REQUIRE(false, "scale: unknown dtype %d", dtype);
+  RLIS_LAUNCH_CHECK("scale");
+  return 0;
+}

@@ -1,0 +1,288 @@
+// Attention over a cached latent: per position the cache holds one row [c | kr], the normed
+// latent c (R numbers) from which every head's keys and values are linear maps, and an
+// optional rotated key part kr (r numbers) that all heads share.
+//
+// The maps are taken to the query side, so that the cache is read as it lies and once for all
+// heads: with k_h = U_h c the score q_h . k_h is (U_h^T q_h) . c, and with v_h = V_h c the
+// output sum_j p_j v_hj is V_h (sum_j p_j c_j).  A step therefore runs
+//   head_linear (q_h -> U_h^T q_h), latent_write (norm, rotation, cache write),
+//   latent_attention (scores and weighted sums of cached rows), head_linear (V_h).
+// Scores, softmax and sums are float32.  A query at position p sees keys at positions <= p and,
+// under a window w, > p - w.  With a sink the softmax's denominator also holds exp(sink[h]):
+// a key with that score (not scaled) and no value.
+#include "common.h"
+#include "tile_mma.h"
+
+#include <math.h>
+
+// ------------------------------------------------------------ one product per head
+// y[t][h][n] = sum_k w[h][n][k] * x[t][h][k]; x rows ldx apart with heads x_head apart, y the
+// same with ldy / y_head; w is (H, N, K) contiguous.  A wave takes 16 tokens x 64 columns.
+template <typename T, typename TO, bool ALIGNED>
+__global__ __launch_bounds__(256) void head_linear_kernel(
+    const T* __restrict__ x, long long ldx, int x_head, const T* __restrict__ w,
+    TO* __restrict__ y, long long ldy, int y_head, int rows, int N, int K) {
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int h = blockIdx.z;
+  const int t0 = (blockIdx.x * 4 + wave) * 16;
+  if (t0 >= rows) return;
+  const int n0 = blockIdx.y * 64;
+  const int ta = min(t0 + lane % 16, rows - 1);
+  const T* a_row = x + (long long)ta * ldx + (long long)h * x_head;
+  const T* b_row[4];
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    const int n = min(n0 + b * 16 + lane % 16, N - 1);
+    b_row[b] = w + ((long long)h * N + n) * K;
+  }
+  mma_f32x4 acc[4];
+  wave_tile_product<T, 4, ALIGNED>(a_row, b_row, K, acc);
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    const int n = n0 + b * 16 + lane % 16;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int t = t0 + (lane / 16) * 4 + i;
+      if (t < rows && n < N) st(y + (long long)t * ldy + (long long)h * y_head + n, acc[b][i]);
+    }
+  }
+}
+
+RLIS_API int rlis_head_linear(const void* x, int dtype, long long ldx, int x_head, const void* w,
+                              void* y, int y_dtype, long long ldy, int y_head, int rows, int H,
+                              int N, int K, hipStream_t stream) {
+  RLIS_REQUIRE(rows >= 0 && H > 0 && N > 0 && K > 0, "head_linear: bad sizes");
+  RLIS_REQUIRE(x_head >= K && y_head >= N && ldx >= (long long)(H - 1) * x_head + K &&
+                   ldy >= (long long)(H - 1) * y_head + N,
+               "head_linear: strides shorter than the heads they hold");
+  RLIS_REQUIRE(H <= 65535 && ceil_div(N, 64) <= 65535, "head_linear: too many heads or columns");
+  if (rows == 0) return 0;
+  dim3 grid(ceil_div(rows, 64), ceil_div(N, 64), H);
+#define LAUNCH(T, TO, AL)                                                                  \
+  head_linear_kernel<T, TO, AL><<<grid, 256, 0, stream>>>((const T*)x, ldx, x_head,        \
+                                                         (const T*)w, (TO*)y, ldy, y_head, \
+                                                         rows, N, K)
+  if (dtype == RLIS_BF16) {
+    const bool al = mma_rows_aligned<bf16_t>(x, ldx, x_head, K) &&
+                    mma_rows_aligned<bf16_t>(w, K, 0, K);
+    if (y_dtype == RLIS_BF16) { if (al) LAUNCH(bf16_t, bf16_t, true); else LAUNCH(bf16_t, bf16_t, false); }
+    else { if (al) LAUNCH(bf16_t, float, true); else LAUNCH(bf16_t, float, false); }
+  } else if (dtype == RLIS_F32) {
+    RLIS_REQUIRE(y_dtype == RLIS_F32, "head_linear: a float32 product has a float32 result");
+    const bool al = mma_rows_aligned<float>(x, ldx, x_head, K) && mma_rows_aligned<float>(w, K, 0, K);
+    if (al) LAUNCH(float, float, true); else LAUNCH(float, float, false);
+  } else {
+    RLIS_REQUIRE(false, "head_linear: unknown dtype %d", dtype);
+  }
+#undef LAUNCH
+  RLIS_LAUNCH_CHECK("head_linear");
+  return 0;
+}
+
+// ------------------------------------------------- norm, rotation and cache write
+// Per token: c = x[:R] / sqrt(mean(x[:R]^2) + eps) * weight goes to the token's cache row, the
+// r numbers behind it are rotated by the token's position (the first rot of them: entry i with
+// entry i + rot/2; the rest pass) and follow c in the row; the last r numbers of every query
+// head are rotated the same way into the head's row of q_out behind its first R columns.
+// x is float32; angles come from float32 tables (positions, rot/2).
+template <typename TX>
+__global__ __launch_bounds__(256) void latent_write_kernel(
+    const float* __restrict__ x, long long ldx, const float* __restrict__ weight, float eps,
+    int R, int r, int rot, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    const int* __restrict__ positions, const int* __restrict__ slots, TX* __restrict__ pages,
+    int write, const TX* __restrict__ q, long long ldq, int q_head, int q_off,
+    TX* __restrict__ q_out, long long ldo, int o_head, int H) {
+  __shared__ float red[4];
+  const int t = blockIdx.x;
+  const int pos = positions[t];
+  const int half = rot / 2;
+  const float* xr = x + (long long)t * ldx;
+  if (write) {
+    TX* row = pages + (long long)slots[t] * (R + r);
+    float ss = 0.f;
+    for (int j = threadIdx.x; j < R; j += 256) ss += xr[j] * xr[j];
+    ss = block_sum<256>(ss, red);
+    const float mult = 1.0f / sqrtf(ss / (float)R + eps);
+    for (int j = threadIdx.x; j < R; j += 256) st(row + j, xr[j] * mult * weight[j]);
+    for (int j = threadIdx.x; j < r; j += 256) {
+      float v = xr[R + j];
+      if (j < rot) {
+        const int i = j < half ? j : j - half;
+        const float c = cos_t[(long long)pos * half + i], s = sin_t[(long long)pos * half + i];
+        const float u = xr[R + i], w = xr[R + i + half];
+        v = j < half ? u * c - w * s : w * c + u * s;
+      }
+      st(row + R + j, v);
+    }
+  }
+  for (int e = threadIdx.x; e < H * r; e += 256) {
+    const int h = e / r, j = e % r;
+    const TX* qh = q + (long long)t * ldq + (long long)h * q_head + q_off;
+    float v = ld(qh + j);
+    if (j < rot) {
+      const int i = j < half ? j : j - half;
+      const float c = cos_t[(long long)pos * half + i], s = sin_t[(long long)pos * half + i];
+      const float u = ld(qh + i), w = ld(qh + i + half);
+      v = j < half ? u * c - w * s : w * c + u * s;
+    }
+    st(q_out + (long long)t * ldo + (long long)h * o_head + R + j, v);
+  }
+}
+
+RLIS_API int rlis_latent_write(const float* x, long long ldx, const float* weight, float eps,
+                               int R, int r, int rot, const float* cos_t, const float* sin_t,
+                               const int* positions, const int* slots, void* pages, int dtype,
+                               int write, const void* q, long long ldq, int q_head, int q_off,
+                               void* q_out, long long ldo, int o_head, int H, int T,
+                               hipStream_t stream) {
+  RLIS_REQUIRE(T >= 0 && R > 0 && r >= 0 && rot >= 0 && rot <= r && rot % 2 == 0 && H > 0,
+               "latent_write: bad sizes R=%d r=%d rot=%d", R, r, rot);
+  RLIS_REQUIRE(rot == 0 || (cos_t && sin_t), "latent_write: a rotation needs its tables");
+  RLIS_REQUIRE(!write || (ldx >= R + r && pages && slots && weight),
+               "latent_write: the cache write needs rows, pages and slots");
+  RLIS_REQUIRE(r == 0 || (q && q_out && q_head >= q_off + r && o_head >= R + r),
+               "latent_write: the rotated query part needs its rows");
+  if (T == 0 || (!write && r == 0)) return 0;
+#define LAUNCH(TX)                                                                            \
+  latent_write_kernel<TX><<<T, 256, 0, stream>>>(x, ldx, weight, eps, R, r, rot, cos_t, sin_t, \
+                                                 positions, slots, (TX*)pages, write,          \
+                                                 (const TX*)q, ldq, q_head, q_off, (TX*)q_out, \
+                                                 ldo, o_head, H)
+  if (dtype == RLIS_F32) LAUNCH(float);
+  else if (dtype == RLIS_BF16) LAUNCH(bf16_t);
+  else RLIS_REQUIRE(false, "latent_write: unknown dtype %d", dtype);
+#undef LAUNCH
+  RLIS_LAUNCH_CHECK("latent_write");
+  return 0;
+}
+
+// --------------------------------------------------------------- attention, vector units
+// One wave per (token, head).  q rows hold per head the D = R + r numbers that meet a cached
+// row; the output per head is sum_j p_j c_j over the first R numbers of the rows.  A lane takes
+// one key of a round of 64 (its whole dot product), then the lanes share the columns of the
+// weighted sum.
+template <typename TX, int CPL>
+__global__ __launch_bounds__(64) void latent_attention_kernel(
+    const TX* __restrict__ q, long long ldq, TX* __restrict__ out, long long ldo,
+    const TX* __restrict__ pages, const int* __restrict__ block_tables, int max_pages,
+    const int* __restrict__ seq_of_token, const int* __restrict__ positions, int H, int R,
+    int D, int page_size, float scale, int window, const float* __restrict__ sink) {
+  extern __shared__ float smem[];
+  float* q_s = smem;                                // D
+  float* p_s = smem + D;                            // 64
+  long long* row_s = (long long*)(p_s + 64);        // 64
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int seq = seq_of_token[t];
+  const int pos = positions[t];
+  const int* table = block_tables + (long long)seq * max_pages;
+  for (int j = lane; j < D; j += 64) q_s[j] = ld(q + (long long)t * ldq + (long long)h * D + j) * scale;
+  __syncthreads();
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  // the sink is a key that every query sees: it opens the running maximum and denominator
+  float m = sink ? sink[h] : -INFINITY;
+  float l = sink ? 1.f : 0.f;
+  float acc[CPL];
+#pragma unroll
+  for (int i = 0; i < CPL; ++i) acc[i] = 0.f;
+  for (int k0 = lo; k0 <= pos; k0 += 64) {
+    const int kpos = k0 + lane;
+    const bool valid = kpos <= pos;
+    const int kp = valid ? kpos : pos;
+    const long long row = ((long long)table[kp / page_size] * page_size + kp % page_size) * D;
+    const TX* c = pages + row;
+    float dot = 0.f;
+    for (int j = 0; j < D; ++j) dot = fmaf(q_s[j], ld(c + j), dot);
+    const float s = valid ? dot : -INFINITY;
+    const float m_new = fmaxf(m, wave_max(s));
+    const float p = valid ? expf(s - m_new) : 0.f;
+    const float corr = (m == -INFINITY) ? 0.f : expf(m - m_new);
+    l = l * corr + wave_sum(p);
+    p_s[lane] = p;
+    row_s[lane] = row;
+    __syncthreads();
+    const int n = min(64, pos - k0 + 1);
+#pragma unroll
+    for (int i = 0; i < CPL; ++i) {
+      const int j = lane + 64 * i;
+      if (j < R) {
+        float a = acc[i] * corr;
+        for (int kk = 0; kk < n; ++kk) a = fmaf(p_s[kk], ld(pages + row_s[kk] + j), a);
+        acc[i] = a;
+      }
+    }
+    __syncthreads();
+    m = m_new;
+  }
+  const float inv_l = 1.0f / l;
+#pragma unroll
+  for (int i = 0; i < CPL; ++i) {
+    const int j = lane + 64 * i;
+    if (j < R) st(out + (long long)t * ldo + (long long)h * R + j, acc[i] * inv_l);
+  }
+}
+
+RLIS_API int rlis_latent_attention(const void* q, int dtype, long long ldq, void* out,
+                                   long long ldo, const void* pages, const int* block_tables,
+                                   int max_pages, const int* seq_of_token, const int* positions,
+                                   int T, int H, int R, int D, int page_size, float scale,
+                                   int window, const float* sink, hipStream_t stream) {
+  RLIS_REQUIRE(T >= 0 && H > 0 && R > 0 && D >= R && page_size > 0 && max_pages > 0,
+               "latent_attention: bad sizes");
+  RLIS_REQUIRE(R <= 1024 && D <= 2048, "latent_attention: latent of %d (row of %d) is too wide",
+               R, D);
+  RLIS_REQUIRE(H <= 65535 && ldq >= (long long)H * D && ldo >= (long long)H * R,
+               "latent_attention: rows shorter than their heads");
+  if (T == 0) return 0;
+  dim3 grid(T, H);
+  const size_t smem = (size_t)D * 4 + 64 * 4 + 64 * 8 + 8;
+  const int cpl = ceil_div(R, 64);
+#define LAUNCH(TX, CPL)                                                                       \
+  latent_attention_kernel<TX, CPL><<<grid, 64, smem, stream>>>(                               \
+      (const TX*)q, ldq, (TX*)out, ldo, (const TX*)pages, block_tables, max_pages,            \
+      seq_of_token, positions, H, R, D, page_size, scale, window, sink)
+#define BY_CPL(TX)                         \
+  do {                                     \
+    if (cpl <= 1) LAUNCH(TX, 1);           \
+    else if (cpl <= 2) LAUNCH(TX, 2);      \
+    else if (cpl <= 4) LAUNCH(TX, 4);      \
+    else if (cpl <= 8) LAUNCH(TX, 8);      \
+    else LAUNCH(TX, 16);                   \
+  } while (0)
+  if (dtype == RLIS_F32) BY_CPL(float);
+  else if (dtype == RLIS_BF16) BY_CPL(bf16_t);
+  else RLIS_REQUIRE(false, "latent_attention: unknown dtype %d", dtype);
+#undef BY_CPL
+#undef LAUNCH
+  RLIS_LAUNCH_CHECK("latent_attention");
+  return 0;
+}
+
+// ----------------------------------------------------------------- sigmoid gate
+// o[t][j] *= sigmoid(g[t][j]) in place for rows ldo / ldg apart, the product in float32 with
+// one rounding.
+template <typename TX>
+__global__ void sigmoid_gate_kernel(TX* __restrict__ o, long long ldo, const TX* __restrict__ g,
+                                    long long ldg, int N, long long total) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const long long t = i / N;
+  const int j = (int)(i % N);
+  TX* p = o + t * ldo + j;
+  st(p, ld(p) / (1.0f + expf(-ld(g + t * ldg + j))));
+}
+
+RLIS_API int rlis_sigmoid_gate(void* o, long long ldo, const void* g, long long ldg, int dtype,
+                               int T, int N, hipStream_t stream) {
+  RLIS_REQUIRE(T >= 0 && N > 0 && ldo >= N && ldg >= N, "sigmoid_gate: bad sizes");
+  const long long total = (long long)T * N;
+  if (total == 0) return 0;
+  const unsigned blocks = (unsigned)ceil_div_ll(total, 256);
+  if (dtype == RLIS_F32)
+    sigmoid_gate_kernel<float><<<blocks, 256, 0, stream>>>((float*)o, ldo, (const float*)g, ldg, N, total);
+  else if (dtype == RLIS_BF16)
+    sigmoid_gate_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)o, ldo, (const bf16_t*)g, ldg, N, total);
+  else
+    RLIS_REQUIRE(false, "sigmoid_gate: unknown dtype %d", dtype);
+  RLIS_LAUNCH_CHECK("sigmoid_gate");
+  return 0;
+}

@@ -1,0 +1,292 @@
+// A routed feed-forward: every token goes through `top` of E small gated units.
+//
+//  * moe_route: from the router's float32 logits z: s = sigmoid(z); choice = s + correction;
+//    experts stand in G equal groups of neighbours, a group's score is the sum of its two
+//    largest choice scores, only experts of the `keep` best groups can be chosen (the others
+//    count as minus infinity); the `top` largest choice scores win (the lower index on a tie);
+//    an expert's weight is its s times `scale`, not renormalised.  One wave per token.
+//  * moe_sort: the step's (token, choice) pairs ordered by expert, every expert's run padded to
+//    whole tiles of rows, so that a tile has one expert.  Decided on the device: nothing waits
+//    for the host.  Which row of its expert's run a pair gets does not move its result: rows of a
+//    tile do not see each other.
+//  * moe_gate_up / moe_down: the units' products on the matrix cores, tile by tile
+//    (tile_mma.h), rows gathered through the sorted list; silu(gate) * up in the epilogue of the
+//    first, the pair's weight in the epilogue of the second.
+//  * moe_combine: a token's pairs added in the order of its choices, plus an optional addend
+//    (a shared unit that every token takes), float32.
+#include "common.h"
+#include "tile_mma.h"
+
+#include <math.h>
+
+// ------------------------------------------------------------------------ route
+constexpr int kRouteMaxPerLane = 8;      // experts up to 64 * 8
+
+__device__ __forceinline__ void wave_argmax(float& v, int& idx) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(v, o, kWave);
+    const int oi = __shfl_xor(idx, o, kWave);
+    if (ov > v || (ov == v && oi < idx)) { v = ov; idx = oi; }
+  }
+}
+
+__global__ __launch_bounds__(64) void moe_route_kernel(
+    const float* __restrict__ z, long long ldz, const float* __restrict__ correction, int E,
+    int G, int keep, int top, float scale, int* __restrict__ chosen, float* __restrict__ weights) {
+  extern __shared__ float sm[];
+  float* choice = sm;            // E
+  float* gscore = sm + E;        // G
+  const int t = blockIdx.x, lane = threadIdx.x;
+  const int per = E / G;
+  for (int e = lane; e < E; e += 64) {
+    const float s = 1.0f / (1.0f + expf(-z[(long long)t * ldz + e]));
+    choice[e] = s + correction[e];
+  }
+  __syncthreads();
+  for (int g = lane; g < G; g += 64) {
+    float a = -INFINITY, b = -INFINITY;       // the group's two largest
+    for (int i = 0; i < per; ++i) {
+      const float c = choice[g * per + i];
+      if (c > a) { b = a; a = c; } else if (c > b) { b = c; }
+    }
+    gscore[g] = per > 1 ? a + b : a;
+  }
+  __syncthreads();
+  // the groups that stay: `keep` rounds of the largest score, lower index on a tie
+  for (int round = 0; round < keep; ++round) {
+    float v = -INFINITY;
+    int idx = 0x7fffffff;
+    for (int g = lane; g < G; g += 64) {
+      const float c = gscore[g];
+      if (c == c && (c > v || (c == v && g < idx)) && c != INFINITY) { v = c; idx = g; }
+    }
+    wave_argmax(v, idx);
+    if (lane == 0 && idx != 0x7fffffff) gscore[idx] = INFINITY;     // marks a kept group
+    __syncthreads();
+  }
+  for (int e = lane; e < E; e += 64)
+    if (gscore[e / per] != INFINITY) choice[e] = -INFINITY;
+  __syncthreads();
+  for (int round = 0; round < top; ++round) {
+    float v = -INFINITY;
+    int idx = 0x7fffffff;
+    for (int e = lane; e < E; e += 64) {
+      const float c = choice[e];
+      if (c > v || (c == v && e < idx && c != -INFINITY)) { v = c; idx = e; }
+    }
+    wave_argmax(v, idx);
+    if (idx == 0x7fffffff) idx = 0;            // fewer experts allowed than asked for
+    if (lane == 0) {
+      chosen[(long long)t * top + round] = idx;
+      const float s = 1.0f / (1.0f + expf(-z[(long long)t * ldz + idx]));
+      weights[(long long)t * top + round] = v == -INFINITY ? 0.f : s * scale;
+      choice[idx] = -INFINITY;
+    }
+    __syncthreads();
+  }
+}
+
+RLIS_API int rlis_moe_route(const float* z, long long ldz, const float* correction, int T, int E,
+                            int G, int keep, int top, float scale, int* chosen, float* weights,
+                            hipStream_t stream) {
+  RLIS_REQUIRE(T >= 0 && E > 0 && G > 0 && E % G == 0 && keep >= 1 && keep <= G && top >= 1,
+               "moe_route: bad sizes E=%d groups=%d keep=%d top=%d", E, G, keep, top);
+  RLIS_REQUIRE(top <= keep * (E / G), "moe_route: %d experts asked of %d allowed", top,
+               keep * (E / G));
+  RLIS_REQUIRE(E <= 64 * 1024 / 8, "moe_route: too many experts");
+  if (T == 0) return 0;
+  moe_route_kernel<<<T, 64, (size_t)(E + G) * 4, stream>>>(z, ldz, correction, E, G, keep, top,
+                                                          scale, chosen, weights);
+  RLIS_LAUNCH_CHECK("moe_route");
+  return 0;
+}
+
+// ------------------------------------------------------------------------- sort
+// sorted[row] = pair (or -1 for padding), tile_expert[tile] = expert (or -1: tile unused).
+// One workgroup.  `tile_rows` rows a tile; `max_tiles` tiles are laid out.
+__global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ chosen, int P,
+                                                        int E, int tile_rows, int max_tiles,
+                                                        int* __restrict__ sorted,
+                                                        int* __restrict__ tile_expert) {
+  extern __shared__ int si[];
+  int* count = si;          // E
+  int* start = si + E;      // E
+  for (int e = threadIdx.x; e < E; e += blockDim.x) count[e] = 0;
+  for (int i = threadIdx.x; i < max_tiles * tile_rows; i += blockDim.x) sorted[i] = -1;
+  for (int i = threadIdx.x; i < max_tiles; i += blockDim.x) tile_expert[i] = -1;
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += blockDim.x) atomicAdd(&count[chosen[p]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int tile = 0;
+    for (int e = 0; e < E; ++e) {
+      start[e] = tile * tile_rows;
+      const int tiles = (count[e] + tile_rows - 1) / tile_rows;
+      for (int i = 0; i < tiles && tile + i < max_tiles; ++i) tile_expert[tile + i] = e;
+      tile += tiles;
+      count[e] = 0;
+    }
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += blockDim.x) {
+    const int e = chosen[p];
+    sorted[start[e] + atomicAdd(&count[e], 1)] = p;
+  }
+}
+
+RLIS_API int rlis_moe_sort(const int* chosen, int P, int E, int tile_rows, int max_tiles,
+                           int* sorted, int* tile_expert, hipStream_t stream) {
+  RLIS_REQUIRE(P >= 0 && E > 0 && tile_rows > 0 && max_tiles >= 0, "moe_sort: bad sizes");
+  RLIS_REQUIRE((long long)max_tiles * tile_rows >= P + (long long)E * (tile_rows - 1) ||
+                   max_tiles >= P,
+               "moe_sort: %d tiles of %d rows may not hold %d pairs of %d experts", max_tiles,
+               tile_rows, P, E);
+  RLIS_REQUIRE(E <= 8192, "moe_sort: too many experts");
+  if (P == 0) return 0;
+  moe_sort_kernel<<<1, 1024, (size_t)E * 8, stream>>>(chosen, P, E, tile_rows, max_tiles, sorted,
+                                                     tile_expert);
+  RLIS_LAUNCH_CHECK("moe_sort");
+  return 0;
+}
+
+// ---------------------------------------------------------------- gate/up product
+// hidden[row][f] = silu(Wg[e][f] . x[token]) * (Wu[e][f] . x[token]) for the sorted rows of a
+// tile; w_gu is (E, 2 F, K) with an expert's gate rows in front of its up rows.  A workgroup of
+// WAVES waves takes 16 * WAVES rows x 32 columns.
+template <typename T, int WAVES, bool ALIGNED>
+__global__ __launch_bounds__(64 * WAVES) void moe_gate_up_kernel(
+    const T* __restrict__ x, long long ldx, const T* __restrict__ w_gu,
+    const int* __restrict__ sorted, const int* __restrict__ tile_expert, int top, int F, int K,
+    T* __restrict__ hidden) {
+  const int e = tile_expert[blockIdx.x];
+  if (e < 0) return;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int row0 = (blockIdx.x * WAVES + wave) * 16;
+  const int f0 = blockIdx.y * 32;
+  const int pair = sorted[row0 + lane % 16];
+  const T* a_row = x + (long long)(pair < 0 ? 0 : pair / top) * ldx;
+  const T* b_row[4];
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    const int f = min(f0 + (b & 1) * 16 + lane % 16, F - 1);
+    b_row[b] = w_gu + (((long long)e * 2 + (b >> 1)) * F + f) * K;      // 0, 1: gate; 2, 3: up
+  }
+  mma_f32x4 acc[4];
+  wave_tile_product<T, 4, ALIGNED>(a_row, b_row, K, acc);
+#pragma unroll
+  for (int b = 0; b < 2; ++b) {
+    const int f = f0 + b * 16 + lane % 16;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = row0 + (lane / 16) * 4 + i;
+      const float g = acc[b][i], u = acc[b + 2][i];
+      if (f < F) st(hidden + (long long)row * F + f, g / (1.0f + expf(-g)) * u);
+    }
+  }
+}
+
+// y[pair][n] = weight[pair] * (Wd[e][n] . hidden[row]); w_d is (E, N, F).  16 * WAVES rows x 64
+// columns a workgroup.
+template <typename T, int WAVES, bool ALIGNED>
+__global__ __launch_bounds__(64 * WAVES) void moe_down_kernel(
+    const T* __restrict__ hidden, const T* __restrict__ w_d, const int* __restrict__ sorted,
+    const int* __restrict__ tile_expert, const float* __restrict__ weights, int N, int F,
+    float* __restrict__ y) {
+  const int e = tile_expert[blockIdx.x];
+  if (e < 0) return;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int row0 = (blockIdx.x * WAVES + wave) * 16;
+  const int n0 = blockIdx.y * 64;
+  const T* a_row = hidden + (long long)(row0 + lane % 16) * F;
+  const T* b_row[4];
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    const int n = min(n0 + b * 16 + lane % 16, N - 1);
+    b_row[b] = w_d + ((long long)e * N + n) * F;
+  }
+  mma_f32x4 acc[4];
+  wave_tile_product<T, 4, ALIGNED>(a_row, b_row, F, acc);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int pair = sorted[row0 + (lane / 16) * 4 + i];
+    if (pair < 0) continue;
+    const float wt = weights[pair];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int n = n0 + b * 16 + lane % 16;
+      if (n < N) y[(long long)pair * N + n] = acc[b][i] * wt;
+    }
+  }
+}
+
+RLIS_API int rlis_moe_experts(const void* x, int dtype, long long ldx, const void* w_gu,
+                              const void* w_d, const int* sorted, const int* tile_expert,
+                              const float* weights, int tile_rows, int max_tiles, int top, int F,
+                              int K, void* hidden, float* y, hipStream_t stream) {
+  RLIS_REQUIRE((tile_rows == 16 || tile_rows == 64) && max_tiles >= 0 && top > 0 && F > 0 && K > 0,
+               "moe_experts: bad sizes");
+  RLIS_REQUIRE(ldx >= K, "moe_experts: row stride shorter than a row");
+  if (max_tiles == 0) return 0;
+  RLIS_REQUIRE(ceil_div(F, 32) <= 65535 && ceil_div(K, 64) <= 65535, "moe_experts: too wide");
+  dim3 g1(max_tiles, ceil_div(F, 32)), g2(max_tiles, ceil_div(K, 64));
+#define LAUNCH(T, WAVES, AL1, AL2)                                                             \
+  do {                                                                                         \
+    moe_gate_up_kernel<T, WAVES, AL1><<<g1, 64 * WAVES, 0, stream>>>(                          \
+        (const T*)x, ldx, (const T*)w_gu, sorted, tile_expert, top, F, K, (T*)hidden);         \
+    moe_down_kernel<T, WAVES, AL2><<<g2, 64 * WAVES, 0, stream>>>(                             \
+        (const T*)hidden, (const T*)w_d, sorted, tile_expert, weights, K, F, y);               \
+  } while (0)
+#define BY_ALIGN(T, WAVES)                                                                    \
+  do {                                                                                        \
+    const bool a1 = mma_rows_aligned<T>(x, ldx, 0, K) && mma_rows_aligned<T>(w_gu, K, 0, K);  \
+    const bool a2 = mma_rows_aligned<T>(hidden, F, 0, F) && mma_rows_aligned<T>(w_d, F, 0, F); \
+    if (a1 && a2) LAUNCH(T, WAVES, true, true);                                               \
+    else if (a1) LAUNCH(T, WAVES, true, false);                                               \
+    else if (a2) LAUNCH(T, WAVES, false, true);                                               \
+    else LAUNCH(T, WAVES, false, false);                                                      \
+  } while (0)
+  if (dtype == RLIS_BF16) {
+    if (tile_rows == 16) BY_ALIGN(bf16_t, 1); else BY_ALIGN(bf16_t, 4);
+  } else if (dtype == RLIS_F32) {
+    if (tile_rows == 16) BY_ALIGN(float, 1); else BY_ALIGN(float, 4);
+  } else {
+    RLIS_REQUIRE(false, "moe_experts: unknown dtype %d", dtype);
+  }
+#undef BY_ALIGN
+#undef LAUNCH
+  RLIS_LAUNCH_CHECK("moe_experts");
+  return 0;
+}
+
+// ---------------------------------------------------------------------- combine
+// out[t][n] = sum over the token's `top` pairs of y[t * top + k][n], in the order of k, plus
+// addend[t][n] when there is one.
+template <typename TA>
+__global__ void moe_combine_kernel(float* __restrict__ out, const float* __restrict__ y,
+                                   const TA* __restrict__ addend, int top, int N, long long total) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const long long t = i / N;
+  const int n = (int)(i % N);
+  float s = 0.f;
+  for (int k = 0; k < top; ++k) s += y[(t * top + k) * N + n];
+  if (addend) s += ld(addend + i);
+  out[i] = s;
+}
+
+RLIS_API int rlis_moe_combine(float* out, const float* y, const void* addend, int addend_dtype,
+                              int T, int top, int N, hipStream_t stream) {
+  RLIS_REQUIRE(T >= 0 && top > 0 && N > 0, "moe_combine: bad sizes");
+  const long long total = (long long)T * N;
+  if (total == 0) return 0;
+  const unsigned blocks = (unsigned)ceil_div_ll(total, 256);
+  if (!addend || addend_dtype == RLIS_F32)
+    moe_combine_kernel<float><<<blocks, 256, 0, stream>>>(out, y, (const float*)addend, top, N, total);
+  else if (addend_dtype == RLIS_BF16)
+    moe_combine_kernel<bf16_t><<<blocks, 256, 0, stream>>>(out, y, (const bf16_t*)addend, top, N, total);
+  else
+    RLIS_REQUIRE(false, "moe_combine: unknown dtype %d", addend_dtype);
+  RLIS_LAUNCH_CHECK("moe_combine");
+  return 0;
+}

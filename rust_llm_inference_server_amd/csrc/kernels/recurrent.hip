@@ -76,7 +76,7 @@ __global__ void tail_update_kernel(float* __restrict__ state, long long state_st
 }
 
 // ------------------------------------------- short causal convolution + SiLU (+ unit norm)
-// y[t][c] = silu(sum_j taps[c][j] * x[t - (K - 1) + j][c]); rows in front of the step come from
+// y[t][c] = silu(bias[c] + sum_j taps[c][j] * x[t - (K - 1) + j][c]) (bias optional); rows in front of the step come from
 // the tail, rows in front of the sequence are the tail's zeros.  Channels [0, unit_channels)
 // are then made unit vectors in groups of unit_group (x / sqrt(sum x^2 + unit_eps)) and those
 // below scaled_channels multiplied by `scale`; the other channels are cut into groups of
@@ -85,10 +85,12 @@ __global__ void tail_update_kernel(float* __restrict__ state, long long state_st
 // tail's) are asked for from addresses that exist, and the value is chosen.
 __device__ __forceinline__ float lanes_sum(float v);
 
+template <typename TO>
 __global__ __launch_bounds__(256) void causal_conv_kernel(
-    float* __restrict__ out, const float* __restrict__ x, long long ldx,
-    const float* __restrict__ taps, int C, int K, const float* __restrict__ state,
-    long long state_stride, const int* __restrict__ seq_of_token, const int* __restrict__ cu,
+    TO* __restrict__ out, const float* __restrict__ x, long long ldx,
+    const float* __restrict__ taps, const float* __restrict__ bias, int C, int K,
+    const float* __restrict__ state, long long state_stride,
+    const int* __restrict__ seq_of_token, const int* __restrict__ cu,
     const int* __restrict__ slots, int unit_channels, int unit_group, int scaled_channels,
     float scale, float unit_eps, int rest_group, int groups) {
   const int t = blockIdx.x;
@@ -118,7 +120,7 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(
     if (v * kWave < width) {                 // the same for the whole wave
       const int off = lane + v * kWave;
       const int c = c0 + (off < width ? off : width - 1);
-      float acc = 0.f;
+      float acc = bias ? bias[c] : 0.f;
       for (int j = 0; j < K; ++j) {
         const int back = R - j;              // how many rows before t
         const bool here = back <= rel;
@@ -139,7 +141,7 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(
 #pragma unroll
   for (int v = 0; v < VPT; ++v) {
     const int off = lane + v * kWave;
-    if (off < width) out[(long long)t * C + c0 + off] = y[v] * mult;
+    if (off < width) st(out + (long long)t * C + c0 + off, y[v] * mult);
   }
 }
 
@@ -852,8 +854,9 @@ RLIS_API int rlis_tail_update(float* state, long long state_stride, const void* 
   return 0;
 }
 
-RLIS_API int rlis_causal_conv(float* out, const float* x, long long ldx, const float* taps, int C,
-                              int K, const float* state, long long state_stride,
+RLIS_API int rlis_causal_conv(void* out, int out_dtype, const float* x, long long ldx, const float* taps,
+                              const float* bias, int C, int K, const float* state,
+                              long long state_stride,
                               const int* seq_of_token, const int* cu, const int* slots, int T,
                               int unit_channels, int unit_group, int scaled_channels, float scale,
                               float unit_eps, int rest_group, hipStream_t stream) {
@@ -871,9 +874,15 @@ RLIS_API int rlis_causal_conv(float* out, const float* x, long long ldx, const f
   const int groups = (unit_channels ? unit_channels / unit_group : 0) +
                      (unit_channels < C ? ceil_div(C - unit_channels, rest_group) : 0);
   RLIS_REQUIRE(ceil_div(groups, 4) <= 65535, "causal_conv: too many groups");
-  causal_conv_kernel<<<dim3(T, ceil_div(groups, 4)), 256, 0, stream>>>(
-      out, x, ldx, taps, C, K, state, state_stride, seq_of_token, cu, slots, unit_channels,
-      unit_group, scaled_channels, scale, unit_eps, rest_group > 0 ? rest_group : 1, groups);
+#define LAUNCH(TO)                                                                           \
+  causal_conv_kernel<TO><<<dim3(T, ceil_div(groups, 4)), 256, 0, stream>>>(                    \
+      (TO*)out, x, ldx, taps, bias, C, K, state, state_stride, seq_of_token, cu, slots,        \
+      unit_channels, unit_group, scaled_channels, scale, unit_eps,                             \
+      rest_group > 0 ? rest_group : 1, groups)
+  if (out_dtype == RLIS_F32) LAUNCH(float);
+  else if (out_dtype == RLIS_BF16) LAUNCH(bf16_t);
+  else RLIS_REQUIRE(false, "causal_conv: unknown dtype %d", out_dtype);
+#undef LAUNCH
   RLIS_LAUNCH_CHECK("causal_conv");
   return 0;
 }
@@ -986,5 +995,104 @@ RLIS_API int rlis_head_norm_gate(void* out, int out_dtype, const float* o, const
   }
 #undef CASE
   RLIS_LAUNCH_CHECK("head_norm_gate");
+  return 0;
+}
+
+
+// ------------------------------------------------------------------ selective scan
+// A state of N numbers per channel with an input-dependent step: per token and channel c
+//   dt = softplus(dt_raw[c] + dt_bias[c]);  S[c][n] <- exp(dt A[c][n]) S[c][n] + dt x[c] B[n];
+//   y[c] = sum_n S[c][n] C[n] + D[c] x[c];  out[c] = y[c] * silu(z[c]),
+// with A = -exp(A_log).  B and C (N numbers each) are the token's, shared by the channels.
+// LPC lanes share a channel, lane `sub` of them holding states n = sub, sub + LPC, ...; a
+// token's sum over n ends with log2(LPC) exchanges between those lanes.  A sequence's tokens
+// are walked in order from the state its slot holds, which is left as after the last one.
+// x (the convolution's output) and the result are in the activation dtype; everything else,
+// the state included, is float32.
+template <typename TO, int NPL, int LPC>
+__global__ __launch_bounds__(256) void selective_scan_kernel(
+    TO* __restrict__ out, long long ldo, const TO* __restrict__ x, long long ldx,
+    const float* __restrict__ dt_raw, long long lddt, const float* __restrict__ dt_bias,
+    const float* __restrict__ bmat, const float* __restrict__ cmat, long long ldbc,
+    const float* __restrict__ z, long long ldz, const float* __restrict__ a_log,
+    const float* __restrict__ dskip, float* __restrict__ state, long long state_stride,
+    const int* __restrict__ cu, const int* __restrict__ slots, int C, int N) {
+  const int s = blockIdx.y;
+  const int gid = blockIdx.x * blockDim.x + threadIdx.x;
+  const int c = gid / LPC, sub = gid % LPC;
+  if (c >= C) return;                 // (LPC divides the wave: a channel's lanes stay together)
+  const int t0 = cu[s], t1 = cu[s + 1];
+  float* S = state + (long long)slots[s] * state_stride + (long long)c * N;
+  float st_[NPL], a[NPL];
+#pragma unroll
+  for (int j = 0; j < NPL; ++j) {
+    const int n = sub + j * LPC;
+    st_[j] = n < N ? S[n] : 0.f;
+    a[j] = n < N ? -expf(a_log[(long long)c * N + n]) : 0.f;
+  }
+  const float bias = dt_bias[c], dsk = dskip[c];
+  for (int t = t0; t < t1; ++t) {
+    const float raw = dt_raw[(long long)t * lddt + c] + bias;
+    const float dt = raw > 20.f ? raw : log1pf(expf(raw));
+    const float xv = ld(x + (long long)t * ldx + c);
+    const float dx = dt * xv;
+    const float* bt = bmat + (long long)t * ldbc;
+    const float* ct = cmat + (long long)t * ldbc;
+    float y = 0.f;
+#pragma unroll
+    for (int j = 0; j < NPL; ++j) {
+      const int n = sub + j * LPC;
+      const int nn = n < N ? n : 0;
+      const float bn = bt[nn], cn = ct[nn];
+      const float v = expf(dt * a[j]) * st_[j] + dx * bn;
+      st_[j] = n < N ? v : 0.f;
+      y = fmaf(st_[j], cn, y);
+    }
+#pragma unroll
+    for (int o = 1; o < LPC; o <<= 1) y += __shfl_xor(y, o, kWave);
+    if (sub == 0) {
+      const float zv = z[(long long)t * ldz + c];
+      st(out + (long long)t * ldo + c, (y + dsk * xv) * (zv / (1.0f + expf(-zv))));
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < NPL; ++j) {
+    const int n = sub + j * LPC;
+    if (n < N) S[n] = st_[j];
+  }
+}
+
+RLIS_API int rlis_selective_scan(void* out, int out_dtype, long long ldo, const void* x,
+                                 long long ldx, const float* dt_raw, long long lddt,
+                                 const float* dt_bias, const float* bmat, const float* cmat,
+                                 long long ldbc, const float* z, long long ldz,
+                                 const float* a_log, const float* dskip, float* state,
+                                 long long state_stride, const int* cu, const int* slots,
+                                 int num_seqs, int C, int N, hipStream_t stream) {
+  RLIS_REQUIRE(num_seqs >= 0 && C > 0 && N > 0, "selective_scan: bad sizes C=%d N=%d", C, N);
+  RLIS_REQUIRE(N <= 1024, "selective_scan: a state of %d numbers per channel is too large", N);
+  RLIS_REQUIRE(ldo >= C && ldx >= C && lddt >= C && ldz >= C && ldbc >= N &&
+                   state_stride >= (long long)C * N,
+               "selective_scan: strides shorter than rows");
+  RLIS_REQUIRE(num_seqs <= 65535, "selective_scan: too many sequences");
+  if (num_seqs == 0) return 0;
+#define LAUNCH(TO, NPL, LPC)                                                                  \
+  selective_scan_kernel<TO, NPL, LPC><<<dim3(ceil_div(C * LPC, 256), num_seqs), 256, 0, stream>>>( \
+      (TO*)out, ldo, (const TO*)x, ldx, dt_raw, lddt, dt_bias, bmat, cmat, ldbc, z, ldz, a_log, dskip,   \
+      state, state_stride, cu, slots, C, N)
+#define BY_N(TO)                                  \
+  do {                                            \
+    if (N <= 16) LAUNCH(TO, 4, 4);                \
+    else if (N <= 32) LAUNCH(TO, 8, 4);           \
+    else if (N <= 64) LAUNCH(TO, 16, 4);          \
+    else if (N <= 256) LAUNCH(TO, 16, 16);        \
+    else LAUNCH(TO, 16, 64);                      \
+  } while (0)
+  if (out_dtype == RLIS_F32) BY_N(float);
+  else if (out_dtype == RLIS_BF16) BY_N(bf16_t);
+  else RLIS_REQUIRE(false, "selective_scan: unknown dtype %d", out_dtype);
+#undef BY_N
+#undef LAUNCH
+  RLIS_LAUNCH_CHECK("selective_scan");
   return 0;
 }

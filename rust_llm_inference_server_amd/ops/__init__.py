@@ -244,6 +244,47 @@ def add_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torc
     return out
 
 
+def add_layernorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor,
+                  bias: torch.Tensor, eps: float, out_dtype: torch.dtype,
+                  rows: Optional[torch.Tensor] = None, write_resid: bool = True,
+                  round_parts: bool = False, delta_scale: float = 1.0) -> torch.Tensor:
+    """``(x - mean) / sqrt(var + eps) * weight + bias`` row by row for
+    ``x = resid + delta_scale * delta``, ``var`` the mean squared deviation; arguments as for
+    ``add_rmsnorm``."""
+    _check(resid, "residual", torch.float32, 2)
+    T, H = resid.shape
+    if not resid.is_contiguous():
+        raise KernelError("add_layernorm: residual must be contiguous")
+    parts = 1 if delta is None else _delta_parts(resid, delta, "add_layernorm")
+    for t, what in ((weight, "weight"), (bias, "bias")):
+        _check(t, f"norm {what}", ndim=1)
+        if t.numel() != H or not t.is_contiguous():
+            raise KernelError(f"add_layernorm: {what} has {t.numel()} entries, rows have {H}")
+    if weight.dtype != bias.dtype:
+        raise KernelError("add_layernorm: weight and bias must share a dtype")
+    if rows is not None:
+        R, rows_ptr, write_resid = rows.numel(), _i32(rows, "rows"), False
+    else:
+        R, rows_ptr = T, None
+    out = torch.empty((R, H), dtype=out_dtype, device=resid.device)
+    lib.call("rlis_add_layernorm", resid.data_ptr(),
+             None if delta is None else delta.data_ptr(), 0 if delta is None else _dt(delta),
+             weight.data_ptr(), bias.data_ptr(), _dt(weight), out.data_ptr(), _DT[out_dtype],
+             rows_ptr, R, H, float(eps), int(bool(write_resid)), parts, T * H,
+             int(bool(round_parts) and delta is not None and delta.dim() > resid.dim()),
+             float(delta_scale), lib.stream_ptr())
+    return out
+
+
+def scale_(x: torch.Tensor, factor: float) -> torch.Tensor:
+    """``x <- x * factor`` in place."""
+    _check(x, "scale")
+    if not x.is_contiguous():
+        raise KernelError("scale: tensor must be contiguous")
+    lib.call("rlis_scale", x.data_ptr(), _dt(x), x.numel(), float(factor), lib.stream_ptr())
+    return x
+
+
 def swiglu(gu: torch.Tensor) -> torch.Tensor:
     """``silu(gu[:, :I]) * gu[:, I:]`` for ``gu`` of shape ``(T, 2 I)``."""
     _check(gu, "gate/up", ndim=2)
@@ -1047,7 +1088,9 @@ def sample_rows(logits: torch.Tensor, keys: torch.Tensor, inv_temps: torch.Tenso
 
 
 from .recurrent import (causal_conv, decay_scan, delta_scan, head_norm_gate,  # noqa: E402,F401
-                        shift_mix, tail_update)
+                        selective_scan, shift_mix, tail_update)
+from .latent import head_linear, latent_attention, latent_write, sigmoid_gate_  # noqa: E402,F401
+from .routed import routed_units, route  # noqa: E402,F401
 
 
 def fill_normal(out: torch.Tensor, seed: int, tensor_index: int, mean: float, std: float) -> None:

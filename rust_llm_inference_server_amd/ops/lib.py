@@ -26,7 +26,18 @@ _SIGNATURES = {
     "rlis_soft_cap": [P, I, L, F, P],
     "rlis_shift_mix": [P, P, I, P, P, L, P, P, P, I, I, I, P],
     "rlis_tail_update": [P, L, P, I, L, I, I, P, P, I, P],
-    "rlis_causal_conv": [P, P, L, P, I, I, P, L, P, P, P, I, I, I, I, F, F, I, P],
+    "rlis_causal_conv": [P, I, P, L, P, P, I, I, P, L, P, P, P, I, I, I, I, F, F, I, P],
+    "rlis_selective_scan": [P, I, L, P, L, P, L, P, P, P, L, P, L, P, P, P, L, P, P, I, I, I, P],
+    "rlis_add_layernorm": [P, P, I, P, P, I, P, I, P, I, I, F, I, I, L, I, F, P],
+    "rlis_scale": [P, I, L, F, P],
+    "rlis_head_linear": [P, I, L, I, P, P, I, L, I, I, I, I, I, P],
+    "rlis_latent_write": [P, L, P, F, I, I, I, P, P, P, P, P, I, I, P, L, I, I, P, L, I, I, I, P],
+    "rlis_latent_attention": [P, I, L, P, L, P, P, I, P, P, I, I, I, I, I, F, I, P, P],
+    "rlis_sigmoid_gate": [P, L, P, L, I, I, I, P],
+    "rlis_moe_route": [P, L, P, I, I, I, I, I, F, P, P, P],
+    "rlis_moe_sort": [P, I, I, I, I, P, P, P],
+    "rlis_moe_experts": [P, I, L, P, P, P, P, P, I, I, I, I, I, P, P, P],
+    "rlis_moe_combine": [P, P, P, I, I, I, I, P],
     "rlis_delta_scan": [P, L, P, P, P, L, P, P, L, P, P, P, L, P, P, I, I, I, I, I, I, P],
     "rlis_decay_scan": [P, P, P, P, P, L, P, P, P, L, P, P, I, I, I, I, P],
     "rlis_head_norm_gate": [P, I, P, P, I, P, I, L, I, I, I, F, P],

@@ -108,12 +108,14 @@ def tail_update(state: torch.Tensor, x: torch.Tensor, channels: int, rows: int, 
 def causal_conv(x: torch.Tensor, taps: torch.Tensor, state: torch.Tensor,
                 seq_of_token: torch.Tensor, cu: torch.Tensor, slots: torch.Tensor, num_seqs: int,
                 unit_channels: int = 0, unit_group: int = 0, scaled_channels: int = 0,
-                scale: float = 1.0, unit_eps: float = 0.0, rest_group: int = 256) -> torch.Tensor:
+                scale: float = 1.0, unit_eps: float = 0.0, rest_group: int = 256,
+                bias: Optional[torch.Tensor] = None,
+                out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
     """``silu`` of the causal convolution over time of the first ``C`` columns of ``x`` (float32)
     with ``taps (C, K)`` (the last column multiplies the current row; the ``K - 1`` rows in
-    front of the step come from ``state``).  Channels below ``unit_channels`` are then made
+    front of the step come from ``state``), plus ``bias (C)`` under the ``silu`` when given.  Channels below ``unit_channels`` are then made
     unit vectors in groups of ``unit_group``: ``y / sqrt(sum y^2 + unit_eps)``, those below
-    ``scaled_channels`` times ``scale``.  Returns ``(T, C)`` float32."""
+    ``scaled_channels`` times ``scale``.  Returns ``(T, C)`` in ``out_dtype`` (float32 arithmetic)."""
     ldx = _rows(x, "causal_conv x", torch.float32)
     C, K = taps.shape
     _vec(taps.reshape(-1), C * K, "causal_conv taps")
@@ -121,8 +123,9 @@ def causal_conv(x: torch.Tensor, taps: torch.Tensor, state: torch.Tensor,
         raise KernelError(f"causal_conv: x has {x.shape[1]} columns, the taps {C} channels")
     T = x.shape[0]
     stride = _state(state, C * (K - 1), "causal_conv")
-    out = torch.empty((T, C), dtype=torch.float32, device=x.device)
-    lib.call("rlis_causal_conv", out.data_ptr(), x.data_ptr(), ldx, taps.data_ptr(), C, K,
+    out = torch.empty((T, C), dtype=out_dtype, device=x.device)
+    lib.call("rlis_causal_conv", out.data_ptr(), _DT[out_dtype], x.data_ptr(), ldx,
+             taps.data_ptr(), None if bias is None else _vec(bias, C, "causal_conv bias"), C, K,
              state.data_ptr(), stride, _meta(seq_of_token, T, "seq_of_token"),
              _meta(cu, num_seqs + 1, "cu"), _meta(slots, num_seqs, "slots"), T,
              int(unit_channels), int(unit_group), int(scaled_channels), float(scale),
@@ -213,5 +216,41 @@ def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, he
     out = torch.empty((T, heads * dv), dtype=out_dtype, device=o.device)
     lib.call("rlis_head_norm_gate", out.data_ptr(), _DT[out_dtype], o.data_ptr(),
              weight.data_ptr(), wstride, gate.data_ptr(), _dt(gate), ldg, T, heads, dv, float(eps),
+             lib.stream_ptr())
+    return out
+
+
+def selective_scan(x: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, b: torch.Tensor,
+                   c: torch.Tensor, z: torch.Tensor, a_log: torch.Tensor, skip: torch.Tensor,
+                   state: torch.Tensor, cu: torch.Tensor, slots: torch.Tensor,
+                   num_seqs: int) -> torch.Tensor:
+    """A state of ``N`` numbers per channel with an input-dependent step, over every sequence's
+    tokens of the step: ``dt = softplus(dt_raw + dt_bias)``,
+    ``S[ch][n] <- exp(dt * A[ch][n]) * S[ch][n] + dt * x[ch] * b[n]`` with ``A = -exp(a_log)``,
+    ``y[ch] = sum_n S[ch][n] * c[n] + skip[ch] * x[ch]``, result ``y * silu(z)``.
+
+    ``x (T, C)`` is in the activation dtype and so is the result; ``dt_raw`` and ``z`` ``(T, C)``
+    and ``b``, ``c`` ``(T, N)`` (column ranges of one matrix) are float32 with contiguous rows;
+    ``a_log (C, N)``; ``state (slots, C * N)`` holds S as [channel][n], float32, and is left as
+    after each sequence's last token."""
+    T, C = x.shape
+    N = a_log.shape[1]
+    ldx = _rows(x, "selective_scan x")
+    lddt = _rows(dt_raw, "selective_scan dt", torch.float32)
+    ldz = _rows(z, "selective_scan z", torch.float32)
+    ldbc = _rows(b, "selective_scan B", torch.float32)
+    if _rows(c, "selective_scan C", torch.float32) != ldbc:
+        raise KernelError("selective_scan: B and C must share a row stride")
+    if dt_raw.shape != (T, C) or z.shape != (T, C) or b.shape != (T, N) or c.shape != (T, N) \
+            or a_log.shape != (C, N):
+        raise KernelError("selective_scan: operand shapes do not match the channels and states")
+    stride = _state(state, C * N, "selective_scan")
+    out = torch.empty((T, C), dtype=x.dtype, device=x.device)
+    lib.call("rlis_selective_scan", out.data_ptr(), _dt(out), C, x.data_ptr(), ldx,
+             dt_raw.data_ptr(), lddt, _vec(dt_bias, C, "selective_scan dt bias"), b.data_ptr(),
+             c.data_ptr(), ldbc, z.data_ptr(), ldz, _vec(a_log.reshape(-1), C * N,
+                                                         "selective_scan A_log"),
+             _vec(skip, C, "selective_scan skip"), state.data_ptr(), stride,
+             _meta(cu, num_seqs + 1, "cu"), _meta(slots, num_seqs, "slots"), num_seqs, C, N,
              lib.stream_ptr())
     return out

@@ -1,12 +1,16 @@
-"""The pre-norm decoder block: ``x += mixer(norm(x)); x += feed_forward(norm(x))``
+"""Decoder blocks.  The pre-norm block: ``x += mixer(norm(x)); x += feed_forward(norm(x))``
 (crates/model/src/llama.rs:264-271).  Which mixer, feed-forward and norms it holds, and under
-which weight names, is given by its parameters, layer by layer."""
+which weight names, is given by its parameters, layer by layer.  The parallel block:
+``x += mixer(h) + feed_forward(h)`` with ``h = norm(x)``, one norm that both sublayers read."""
 from __future__ import annotations
 
 from typing import Any, Dict, List
 
+import torch
+
 from .base import (Block, BuildContext, CacheBinding, ResidualStream, TensorSpec,
                    create, join, normed, register, tensor_specs)
+from .. import ops
 
 
 @register("block", "prenorm")
@@ -53,3 +57,45 @@ class PreNormBlock(Block):
         if self.feed_forward is not None:
             stream.add(self.feed_forward.forward(
                 normed(self.ffn_norm, stream, self.feed_forward), step), m)
+
+
+@register("block", "parallel")
+class ParallelBlock(Block):
+    """Parameters: ``mixer``, ``feed_forward`` (None: the mixer alone), ``norm`` (PartSpecs) and
+    ``names``: the weight-name suffix of each under the block's prefix.  The two sublayers'
+    outputs are added in float32 and join the stream as one delta."""
+
+    _SLOTS = (("norm", "norm"), ("mixer", "mixer"), ("feed_forward", "feed_forward"))
+
+    @classmethod
+    def _slots(cls, params: Dict[str, Any]):
+        return cls._SLOTS[:2] if params.get("feed_forward") is None else cls._SLOTS
+
+    @classmethod
+    def tensor_specs(cls, params: Dict[str, Any], prefix: str) -> List[TensorSpec]:
+        out: List[TensorSpec] = []
+        for slot, category in cls._slots(params):
+            out += tensor_specs(category, params[slot], join(prefix, params["names"][slot]))
+        return out
+
+    def __init__(self, params: Dict[str, Any], prefix: str, ctx: BuildContext):
+        super().__init__(params, prefix, ctx)
+        built = {slot: create(category, params[slot], join(prefix, params["names"][slot]), ctx)
+                 for slot, category in self._slots(params)}
+        self.norm, self.mixer = built["norm"], built["mixer"]
+        self.feed_forward = built.get("feed_forward")
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(p.graph_safe for p in (self.norm, self.mixer, self.feed_forward)
+                   if p is not None)
+
+    def forward(self, stream: ResidualStream, step: Any, binding: CacheBinding) -> None:
+        h = self.norm.forward(stream)
+        mixed = self.mixer.forward(h, step, binding)
+        if self.feed_forward is None:
+            stream.add(mixed)
+            return
+        fed = self.feed_forward.forward(h, step)
+        mixed, fed = (d if isinstance(d, torch.Tensor) else d.run() for d in (mixed, fed))
+        stream.add(ops.weighted_sum(mixed, 1.0, fed, 1.0, round_parts=stream.round_parts))

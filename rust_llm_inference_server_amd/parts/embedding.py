@@ -41,7 +41,8 @@ class TokenEmbedding(Embedding):
 class LinearHead(Head):
     """Parameters: ``vocab_size``, ``hidden_size``, ``tied_to`` (name of the tensor to share,
     or None for a weight of its own at ``prefix.weight``; ``weight_name`` names it otherwise,
-    "" for the prefix itself); optional ``soft_cap`` c: logits become ``c * tanh(logits / c)``."""
+    "" for the prefix itself); optional ``scale`` (the float32 logits are multiplied by it) and
+    ``soft_cap`` c: logits become ``c * tanh(logits / c)``."""
 
     graph_safe = True
 
@@ -60,9 +61,12 @@ class LinearHead(Head):
                                or join(prefix, params.get("weight_name", "weight")))
         cap = params.get("soft_cap")
         self.soft_cap = float(cap) if cap else None
+        self.scale = float(params.get("scale", 1.0))
 
     def forward(self, x: Any) -> torch.Tensor:
         logits = project(x, self.weight, torch.float32)
+        if self.scale != 1.0:
+            ops.scale_(logits, self.scale)
         if self.soft_cap is not None:
             ops.soft_cap_(logits, self.soft_cap)
         return logits

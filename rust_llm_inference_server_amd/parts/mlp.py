@@ -1,4 +1,4 @@
-"""SwiGLU feed-forward: ``down(silu(gate(x)) * up(x))`` with three bias-free projections
+"""Feed-forwards.  SwiGLU: ``down(silu(gate(x)) * up(x))`` with three bias-free projections
 (crates/model/src/layers.rs:156-187).  Gate and up run as one product over the row-concatenated
 weights; ``silu`` and the product are 32-bit with one rounding."""
 from __future__ import annotations
@@ -90,3 +90,74 @@ class ClampedGLU(FeedForward):
         gu = project(x, self.w_gate_up, self.act_dtype)
         hidden = ops.clamped_glu(gu, self.limit, self.alpha)
         return ops.pending_linear(hidden, self.w_down, self.act_dtype)
+
+
+@register("feed_forward", "routed_swiglu")
+class RoutedSwiGLU(FeedForward):
+    """A mixture of small SwiGLU units of which every token takes ``top``, and optionally a
+    shared unit that every token takes.
+
+    Parameters: ``hidden_size``, ``expert_size`` (an expert's inner width), ``experts``,
+    ``top``, ``groups`` and ``keep`` (experts stand in ``groups`` equal groups of neighbours;
+    only those of the ``keep`` groups with the largest sum of their two best choice scores
+    can be chosen), ``scale`` (multiplies the chosen experts' scores, which are not
+    renormalised), ``shared_size`` (None: no shared unit).
+
+    Tensors under the prefix: ``router`` (experts, W), ``correction`` (experts: added to the
+    sigmoid scores for the choice only), ``e<i>.gate|up`` (F, W), ``e<i>.down`` (W, F),
+    ``shared.gate|up|down``.  Router logits, scores and the choice are float32."""
+
+    graph_safe = True
+
+    @classmethod
+    def tensor_specs(cls, params: Dict[str, Any], prefix: str) -> List[TensorSpec]:
+        W, F, E = params["hidden_size"], params["expert_size"], params["experts"]
+        out: List[TensorSpec] = []
+        for e in range(E):
+            out += [TensorSpec(join(prefix, f"e{e}.gate"), (F, W)),
+                    TensorSpec(join(prefix, f"e{e}.up"), (F, W)),
+                    TensorSpec(join(prefix, f"e{e}.down"), (W, F))]
+        out += [TensorSpec(join(prefix, "router"), (E, W), std=0.5),
+                TensorSpec(join(prefix, "correction"), (E,), std=0.1)]
+        S = params.get("shared_size")
+        if S:
+            out += [TensorSpec(join(prefix, "shared.gate"), (S, W)),
+                    TensorSpec(join(prefix, "shared.up"), (S, W)),
+                    TensorSpec(join(prefix, "shared.down"), (W, S))]
+        return out
+
+    def __init__(self, params: Dict[str, Any], prefix: str, ctx: BuildContext):
+        super().__init__(params, prefix, ctx)
+        E = self.experts = int(params["experts"])
+        self.top, self.groups, self.keep = int(params["top"]), int(params["groups"]), int(params["keep"])
+        self.scale = float(params["scale"])
+        if E % self.groups or not 1 <= self.keep <= self.groups \
+                or not 1 <= self.top <= self.keep * (E // self.groups):
+            raise ValueError(f"routed_swiglu: {E} experts in {self.groups} groups, {self.keep} "
+                             f"kept, {self.top} chosen do not fit")
+        pop = lambda n: ctx.weights.pop(join(prefix, n))
+        self.act_dtype = ctx.act_dtype
+        to = lambda t: t.to(ctx.act_dtype)
+        # per expert the gate rows in front of the up rows; all experts in one tensor
+        self.w_gate_up = torch.stack([torch.cat([to(pop(f"e{e}.gate")), to(pop(f"e{e}.up"))], dim=0)
+                                      for e in range(E)]).contiguous()
+        self.w_down = torch.stack([to(pop(f"e{e}.down")) for e in range(E)]).contiguous()
+        self.w_router = ctx.take(join(prefix, "router"))
+        self.correction = ctx.take(join(prefix, "correction")).to(torch.float32).contiguous()
+        self.w_shared_gate_up = self.w_shared_down = None
+        if params.get("shared_size"):
+            gate, up = pop("shared.gate"), pop("shared.up")
+            if gate.dtype != up.dtype:
+                gate, up = gate.to(torch.float32), up.to(torch.float32)
+            self.w_shared_gate_up = torch.cat([gate, up], dim=0).contiguous()
+            self.w_shared_down = ctx.take(join(prefix, "shared.down"))
+
+    def forward(self, x: torch.Tensor, step: Any) -> torch.Tensor:
+        logits = ops.linear(x, self.w_router, torch.float32)
+        chosen, weights = ops.route(logits, self.correction, self.groups, self.keep, self.top,
+                                    self.scale)
+        shared = None
+        if self.w_shared_gate_up is not None:
+            shared = ops.linear(ops.linear_swiglu(x, self.w_shared_gate_up), self.w_shared_down,
+                                self.act_dtype)
+        return ops.routed_units(x, self.w_gate_up, self.w_down, chosen, weights, shared)

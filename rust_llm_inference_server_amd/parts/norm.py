@@ -1,7 +1,12 @@
-"""RMSNorm: ``y = x * rsqrt(mean(x^2) + eps) * w`` over the hidden axis; the weight multiplies
+"""Norms over the hidden axis.
+
+RMSNorm: ``y = x * rsqrt(mean(x^2) + eps) * w``; the weight multiplies
 directly, not as ``1 + w`` (crates/model/src/layers.rs:103-122, 141-146), unless the model
 stores its weights around zero (``weight_offset`` 1: ``y = ... * (1 + w)``).  The input is the
-32-bit residual stream; statistics and both multiplies are 32-bit, one rounding at the store."""
+32-bit residual stream; statistics and both multiplies are 32-bit, one rounding at the store.
+
+LayerNorm: ``y = (x - mean) / sqrt(var + eps) * w + b`` with ``var`` the mean squared
+deviation from the mean; the same input, the same precision."""
 from __future__ import annotations
 
 from typing import Any, Dict, List, Optional
@@ -73,3 +78,43 @@ class RMSNorm(Norm):
         if rows is None:
             stream.x, stream.pending = total, None
         return y
+
+
+@register("norm", "layernorm")
+class LayerNorm(Norm):
+    """Parameters: ``size``, ``eps``; optional ``weight_name`` and ``bias_name`` (the tensors'
+    names under the prefix, "weight" and "bias" by default; "" for the prefix itself)."""
+
+    graph_safe = True
+
+    @classmethod
+    def _names(cls, params: Dict[str, Any], prefix: str):
+        return (join(prefix, params.get("weight_name", "weight")),
+                join(prefix, params.get("bias_name", "bias")))
+
+    @classmethod
+    def tensor_specs(cls, params: Dict[str, Any], prefix: str) -> List[TensorSpec]:
+        w, b = cls._names(params, prefix)
+        return [TensorSpec(w, (params["size"],), init="ones_normal"),
+                TensorSpec(b, (params["size"],))]
+
+    def __init__(self, params: Dict[str, Any], prefix: str, ctx: BuildContext):
+        super().__init__(params, prefix, ctx)
+        self.eps = float(params["eps"])
+        w, b = self._names(params, prefix)
+        self.weight, self.bias = ctx.take(w), ctx.take(b)
+        if self.weight.dtype != self.bias.dtype:
+            self.weight, self.bias = (t.to(torch.float32).contiguous()
+                                      for t in (self.weight, self.bias))
+        self.out_dtype = ctx.act_dtype
+
+    def forward(self, stream: ResidualStream) -> torch.Tensor:
+        delta, scale = stream.take_delta()
+        return ops.add_layernorm(stream.x, delta, self.weight, self.bias, self.eps,
+                                 self.out_dtype, round_parts=stream.round_parts,
+                                 delta_scale=scale)
+
+    def forward_rows(self, stream: ResidualStream, rows: torch.Tensor) -> torch.Tensor:
+        return ops.add_layernorm(stream.x, stream.delta(), self.weight, self.bias, self.eps,
+                                 self.out_dtype, rows=rows, round_parts=stream.round_parts,
+                                 delta_scale=stream.pending_scale)

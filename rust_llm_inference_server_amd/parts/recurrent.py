@@ -16,6 +16,10 @@ leave the state as after the step's last token.  What enters a recurrence (decay
 sizes, unit norms, the state itself) is float32 in either activation dtype; the projections
 that feed it store float32 results.
 
+``selective_scan`` (Mamba): the input passes a short causal convolution and SiLU; a state of N
+numbers per channel decays by ``exp(dt A)`` with a step ``dt`` that the token chooses, takes
+``dt x B`` and is read with ``C``; the result is gated by ``silu(z)``.
+
 ``parallel``: two mixers read the same input, and their outputs meet as a weighted sum in
 float32.  Each keeps what it keeps: the pages of the one that asks for a cache, the state
 bytes of both, one after the other.
@@ -202,6 +206,69 @@ class GatedDelta(Mixer):
                            self.dt_bias, S, cu, slots, n, H, G, d, dv)
         y = ops.head_norm_gate(o, self.norm, p[:, c["g"]:c["g"] + H * dv], H, dv, self.eps,
                                self.act_dtype)
+        return ops.pending_linear(y, self.w_o, self.act_dtype)
+
+
+# ------------------------------------------------------------------------ selective scan
+@register("mixer", "selective_scan")
+class SelectiveScan(Mixer):
+    """Parameters: ``hidden_size``, ``inner`` (channels), ``state`` (numbers per channel),
+    ``dt_rank``, ``conv`` (taps).
+
+    Tensors under the prefix: ``in`` (2 * inner, W): x in front of z; ``conv`` (inner, taps)
+    and ``conv.b`` (inner); ``x`` (dt_rank + 2 * state, inner): the step's low-rank input, B
+    and C; ``dt`` (inner, dt_rank) and ``dt.b`` (inner); ``A_log`` (inner, state); ``D``
+    (inner); ``o`` (W, inner).
+
+    Per token and channel: ``dt = softplus(W_dt low + dt.b)``, ``S <- exp(dt A) S + dt x B``
+    with ``A = -exp(A_log)``, ``y = S . C + D x``, result ``y * silu(z)``.  The state slot holds
+    the last ``conv - 1`` inputs of the convolution and S, float32; steps, decays and the state
+    are float32 in either activation dtype."""
+
+    graph_safe = True
+
+    @classmethod
+    def tensor_specs(cls, params: Dict[str, Any], prefix: str) -> List[TensorSpec]:
+        W, C, N = params["hidden_size"], params["inner"], params["state"]
+        rank, taps = params["dt_rank"], params["conv"]
+        return [TensorSpec(join(prefix, "in"), (2 * C, W)),
+                TensorSpec(join(prefix, "conv"), (C, taps), std=0.3),
+                TensorSpec(join(prefix, "conv.b"), (C,)),
+                TensorSpec(join(prefix, "x"), (rank + 2 * N, C)),
+                TensorSpec(join(prefix, "dt"), (C, rank), std=0.3),
+                TensorSpec(join(prefix, "dt.b"), (C,), std=0.5),
+                TensorSpec(join(prefix, "A_log"), (C, N), std=0.5),
+                TensorSpec(join(prefix, "D"), (C,), init="ones_normal"),
+                TensorSpec(join(prefix, "o"), (W, C))]
+
+    def __init__(self, params: Dict[str, Any], prefix: str, ctx: BuildContext):
+        super().__init__(params, prefix, ctx)
+        self.channels, self.states = int(params["inner"]), int(params["state"])
+        self.rank, self.taps = int(params["dt_rank"]), int(params["conv"])
+        if not 1 <= self.taps <= 16:
+            raise ValueError(f"selective_scan: {self.taps} taps (1 to 16)")
+        take = lambda n: ctx.take(join(prefix, n))
+        self.w_in, self.w_x, self.w_dt, self.w_o = take("in"), take("x"), take("dt"), take("o")
+        self.conv_w, self.conv_b = _f32(take("conv")), _f32(take("conv.b"))
+        self.dt_bias, self.a_log, self.skip = _f32(take("dt.b")), _f32(take("A_log")), _f32(take("D"))
+        self.act_dtype = ctx.act_dtype
+
+    def state_bytes(self) -> int:
+        return 4 * ((self.taps - 1) * self.channels + self.channels * self.states)
+
+    def forward(self, x: torch.Tensor, step: Any, binding: CacheBinding) -> Any:
+        C, N, rank = self.channels, self.states, self.rank
+        tail, S = _state_views(binding, (self.taps - 1) * C)
+        cu, slots, n = step.cu_seqlens, step.state_slots, step.num_seqs
+        xz = ops.linear_f32(x, self.w_in)                                  # (T, x | z)
+        xc = ops.causal_conv(xz, self.conv_w, tail, step.seq_of_token, cu, slots, n,
+                             bias=self.conv_b, out_dtype=self.act_dtype)
+        ops.tail_update(tail, xz, C, self.taps - 1, cu, slots, n)
+        low = ops.linear_f32(xc, self.w_x)                                 # (T, dt | B | C)
+        dt_raw = ops.linear(low[:, :rank], self.w_dt, torch.float32)
+        y = ops.selective_scan(xc, dt_raw, self.dt_bias, low[:, rank:rank + N],
+                               low[:, rank + N:rank + 2 * N], xz[:, C:], self.a_log, self.skip,
+                               S, cu, slots, n)
         return ops.pending_linear(y, self.w_o, self.act_dtype)
 
 

@@ -42,20 +42,30 @@ def inverse_frequencies(rot_dim: int, theta: float, scaling: Optional[Dict[str, 
 @register("position", "rope")
 class RotaryEmbedding(PositionEncoding):
     """Parameters: ``rot_dim`` (rotated width, at most the head size), ``theta``, ``scaling``
-    (None or the llama3 fields).  Holds ``cos``/``sin`` float32 ``(max_positions, rot/2)``."""
+    (None or the llama3 fields).  Holds ``cos``/``sin`` float32 ``(max_positions, rot/2)``.
+    Optional ``precise``: frequencies, angles, cosines and sines are made in double precision
+    and rounded once to float32 (without it they are float32 from the start, as the reference
+    makes them)."""
 
     def __init__(self, params: Dict[str, Any], prefix: str, ctx: BuildContext):
         super().__init__(params, prefix, ctx)
         rot = int(params["rot_dim"])
         if rot % 2:
             raise ValueError(f"position encoding 'rope': rot_dim {rot} must be even")
-        inv = inverse_frequencies(rot, params["theta"], params.get("scaling"))
-        pos = torch.arange(ctx.max_positions, dtype=torch.float32).reshape(-1, 1)
+        if params.get("precise"):
+            if params.get("scaling"):
+                raise ValueError("position encoding 'rope': 'precise' has no frequency scaling")
+            f64 = torch.float64
+            inv = float(params["theta"]) ** (-torch.arange(0, rot, 2, dtype=f64) / rot)
+            pos = torch.arange(ctx.max_positions, dtype=f64).reshape(-1, 1)
+        else:
+            inv = inverse_frequencies(rot, params["theta"], params.get("scaling"))
+            pos = torch.arange(ctx.max_positions, dtype=torch.float32).reshape(-1, 1)
         angles = pos * inv.reshape(1, -1)
         self.rot_dim = rot
-        self.inv_freq = inv
-        self.cos = torch.cos(angles).to(ctx.device).contiguous()
-        self.sin = torch.sin(angles).to(ctx.device).contiguous()
+        self.inv_freq = inv.to(torch.float32)
+        self.cos = torch.cos(angles).to(torch.float32).to(ctx.device).contiguous()
+        self.sin = torch.sin(angles).to(torch.float32).to(ctx.device).contiguous()
         self.max_positions = ctx.max_positions
 
 
