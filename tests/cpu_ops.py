@@ -87,12 +87,13 @@ def tail_update(state, x, channels, rows, cu, slots, num_seqs):
 
 
 def causal_conv(x, taps, state, seq_of_token, cu, slots, num_seqs, unit_channels=0, unit_group=0,
-                scaled_channels=0, scale=1.0, unit_eps=0.0, rest_group=256):
+                scaled_channels=0, scale=1.0, unit_eps=0.0, rest_group=256, bias=None,
+                out_dtype=torch.float32):
     C, K = taps.shape
     out = torch.empty((x.shape[0], C), dtype=torch.float32)
     for t0, t1, slot in _seqs(cu, slots, num_seqs):
         both = torch.cat([state[slot, :C * (K - 1)].reshape(K - 1, C), x[t0:t1, :C].float()], dim=0)
-        acc = torch.zeros(t1 - t0, C)
+        acc = torch.zeros(t1 - t0, C) if bias is None else bias.reshape(1, C).repeat(t1 - t0, 1)
         for j in range(K):
             acc += both[j:j + t1 - t0] * taps[:, j]
         out[t0:t1] = acc / (1.0 + torch.exp(-acc))
@@ -101,7 +102,133 @@ def causal_conv(x, taps, state, seq_of_token, cu, slots, num_seqs, unit_channels
         y = y / torch.sqrt((y * y).sum(-1, keepdim=True) + unit_eps)
         out[:, :unit_channels] = y.reshape(x.shape[0], unit_channels)
         out[:, :scaled_channels] *= scale
+    return out.to(out_dtype)
+
+
+def selective_scan(x, dt_raw, dt_bias, b, c, z, a_log, skip, state, cu, slots, num_seqs):
+    T, C = x.shape
+    N = a_log.shape[1]
+    out = torch.empty((T, C), dtype=torch.float32)
+    A = -torch.exp(a_log)
+    dt = torch.nn.functional.softplus(dt_raw + dt_bias)
+    xf = x.float()
+    for t0, t1, slot in _seqs(cu, slots, num_seqs):
+        S = state[slot, :C * N].reshape(C, N).clone()
+        for t in range(t0, t1):
+            S = torch.exp(dt[t].reshape(C, 1) * A) * S + (dt[t] * xf[t]).reshape(C, 1) * b[t]
+            y = S @ c[t] + skip * xf[t]
+            out[t] = y * (z[t] / (1.0 + torch.exp(-z[t])))
+        state[slot, :C * N] = S.reshape(-1)
+    return out.to(x.dtype)
+
+
+# ---- attention over a cached latent --------------------------------------------------------
+def add_layernorm(resid, delta, weight, bias, eps, out_dtype, rows=None, write_resid=True,
+                  round_parts=False, delta_scale=1.0):
+    if delta is not None and delta.dim() == 3:
+        delta = delta.sum(0)
+    x = resid if delta is None else resid + delta_scale * delta.to(torch.float32)
+    if rows is not None:
+        x = x[rows.long()]
+    elif delta is not None and write_resid:
+        resid.copy_(x)
+    mean = x.mean(dim=-1, keepdim=True)
+    var = ((x - mean) ** 2).mean(dim=-1, keepdim=True)
+    return ((x - mean) / torch.sqrt(var + eps) * weight.float() + bias.float()).to(out_dtype)
+
+
+def scale_(x, factor):
+    x.mul_(factor)
+    return x
+
+
+def head_linear(x, w, x_head, out=None, out_head=None, out_dtype=None):
+    H, N, K = w.shape
+    T = x.shape[0]
+    if out is None:
+        out_head, out = N, torch.empty((T, H * N), dtype=out_dtype or x.dtype)
+    for h in range(H):
+        out[:, h * out_head:h * out_head + N] = \
+            (x[:, h * x_head:h * x_head + K].float() @ w[h].float().t()).to(out.dtype)
     return out
+
+
+def _turned(v, pos, cos, sin, dims):
+    half = dims // 2
+    c, s = cos[pos.long()], sin[pos.long()]
+    while c.dim() < v.dim():
+        c, s = c.unsqueeze(1), s.unsqueeze(1)
+    a, b = v[..., :half], v[..., half:dims]
+    return torch.cat([a * c - b * s, b * c + a * s, v[..., dims:]], dim=-1)
+
+
+def latent_write(x, weight, eps, rank, rot_width, rot_dims, cos, sin, positions, slots, pages, q,
+                 q_head, q_out, heads):
+    D = rank + rot_width
+    if x is not None:
+        lat = x[:, :rank]
+        row = lat / torch.sqrt((lat * lat).mean(-1, keepdim=True) + eps) * weight
+        if rot_width:
+            kr = x[:, rank:D]
+            row = torch.cat([row, _turned(kr, positions, cos, sin, rot_dims) if rot_dims else kr], -1)
+        ps = pages.shape[1]
+        for t in range(x.shape[0]):
+            pages[int(slots[t]) // ps, int(slots[t]) % ps] = row[t].to(pages.dtype)
+    if rot_width:
+        T = q.shape[0]
+        qr = q.float().reshape(T, heads, q_head)[..., q_head - rot_width:]
+        if rot_dims:
+            qr = _turned(qr, positions, cos, sin, rot_dims)
+        q_out.reshape(T, heads, D)[..., rank:] = qr.to(q_out.dtype)
+
+
+def latent_attention(q, pages, block_tables, seq_of_token, positions, heads, rank, scale,
+                     window=None, sink=None):
+    T = q.shape[0]
+    ps, D = pages.shape[1], pages.shape[2]
+    qf = q.float().reshape(T, heads, D)
+    out = torch.zeros(T, heads, rank)
+    for t in range(T):
+        table = block_tables[int(seq_of_token[t])].tolist()
+        pos = int(positions[t])
+        lo = max(0, pos - window + 1) if window else 0
+        rows = torch.stack([pages[table[p // ps], p % ps] for p in range(lo, pos + 1)]).float()
+        s = (qf[t] @ rows.t()) * scale                                    # (heads, keys)
+        if sink is not None:
+            s = torch.cat([s, sink.reshape(heads, 1)], dim=1)
+        p = torch.softmax(s, dim=1)[:, :rows.shape[0]]
+        out[t] = p @ rows[:, :rank]
+    return out.reshape(T, heads * rank).to(q.dtype)
+
+
+def sigmoid_gate_(o, g):
+    o.copy_((o.float() * torch.sigmoid(g.float())).to(o.dtype))
+    return o
+
+
+# ---- routed feed-forward -----------------------------------------------------------------
+def route(logits, correction, groups, keep, top, scale):
+    T, E = logits.shape
+    s = torch.sigmoid(logits)
+    choice = (s + correction).reshape(T, groups, E // groups)
+    score = choice.topk(min(2, E // groups), dim=-1).values.sum(-1)
+    kept = torch.zeros(T, groups, dtype=torch.bool)
+    kept.scatter_(1, score.topk(keep, dim=-1).indices, True)
+    choice = choice.masked_fill(~kept.unsqueeze(-1), float("-inf")).reshape(T, E)
+    chosen = choice.topk(top, dim=-1).indices
+    return chosen.to(torch.int32), (s.gather(1, chosen) * scale).float()
+
+
+def routed_units(x, w_gate_up, w_down, chosen, weights, addend=None):
+    T, W = x.shape
+    F = w_gate_up.shape[1] // 2
+    out = torch.zeros(T, W)
+    for t in range(T):
+        for e, wt in zip(chosen[t].tolist(), weights[t].tolist()):
+            gu = w_gate_up[e].float() @ x[t].float()
+            hidden = (gu[:F] / (1.0 + torch.exp(-gu[:F])) * gu[F:]).to(x.dtype).float()
+            out[t] += wt * (w_down[e].float() @ hidden)
+    return out if addend is None else out + addend.float()
 
 
 def delta_scan(q, k, v, b_raw, a_raw, a_log, dt_bias, state, cu, slots, num_seqs, heads,
@@ -269,6 +396,8 @@ def install(monkeypatch) -> None:
                  "pending_linear", "can_fuse_norm_linear", "rope_kv_write", "rope_attention",
                  "copy_pages", "attention_planner", "paged_attention", "sample_rows",
                  "clamped_glu", "weighted_sum", "linear_f32", "soft_cap_", "shift_mix", "tail_update",
-                 "causal_conv", "delta_scan", "decay_scan", "head_norm_gate"):
+                 "causal_conv", "delta_scan", "decay_scan", "head_norm_gate", "selective_scan",
+                 "add_layernorm", "scale_", "head_linear", "latent_write", "latent_attention",
+                 "sigmoid_gate_", "route", "routed_units"):
         monkeypatch.setattr(ops, name, globals()[name])
     monkeypatch.setattr(runner, "default_device", lambda: torch.device("cpu"))
