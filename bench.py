@@ -43,7 +43,10 @@ delta rule, clamped gated unit; random weights) at the width, depth, feed-forwar
 vocabulary and attention heads of a Llama preset, beside that preset itself: a prefill of
 ``--prefill-tokens`` tokens in one step, and decode steps at batch 8 and 64 after 512-token
 prompts, each with the bytes a step has to read (weights once, the live requests' cache, and
-for Gipotar their state slots read and written) as a fraction of the HBM rate."""
+for Gipotar their state slots read and written) as a fraction of the HBM rate.
+``--design bekunex`` (or ``gipotar,bekunex``) times the Bekunex design that way (attention over
+a cached latent, selective scan, a routed feed-forward; of the experts' weights a step counts
+those that its tokens reach on average, and of a windowed cache the window)."""
 import argparse
 import copy
 import json
@@ -203,6 +206,42 @@ def gipotar_like(cfg: dict) -> dict:
                        for i in range(cfg["num_hidden_layers"])]}
 
 
+def bekunex_like(cfg: dict) -> dict:
+    """A Bekunex configuration at the sizes of a Llama preset: the same width, depth, vocabulary
+    and head count; layers cycle through attention over a cached latent with a rotated key part
+    (latent of 512, rotated part of 64), a selective scan (2 x width channels, 16 states), the
+    windowed kind with sink and gate (window 1,024) and a reader of that layer's latents; every
+    layer has 32 experts of an eighth of the preset's feed-forward width, of which a token takes
+    six out of two of four groups, and a shared unit of a quarter of it: as many active
+    feed-forward weights per token as the preset has."""
+    W, d, H = cfg["hidden_size"], cfg["head_dim"], cfg["num_attention_heads"]
+    ff = cfg["intermediate_size"]
+    mlp = {"kind": "moe", "expert": {"ff": ff // 8},
+           "router": {"experts": 32, "groups": {"count": 4, "keep": 2}, "scale": 2.5, "top": 6},
+           "shared": {"ff": ff // 4}}
+    full = {"type": "latent_attention", "mlp": mlp,
+            "mixer": {"heads": H, "dim": d, "rot_dim": 64,
+                      "rot": {"dims": 64, "base": cfg["rope_theta"]}, "vdim": d, "kv_rank": 512,
+                      "scale": (d + 64) ** -0.5}}
+    scan = {"type": "mamba1", "mlp": mlp,
+            "mixer": {"inner": 2 * W, "state": 16, "dt_rank": max(1, W // 16), "conv": 4}}
+
+    def windowed(kv_from):
+        m = {"heads": H, "dim": d, "vdim": d, "kv_rank": 512, "mask": {"size": 1024},
+             "scale": d ** -0.5}
+        if kv_from is not None:
+            m["kv_from"] = kv_from
+        return {"type": "latent_attention_2", "mlp": mlp, "mixer": m}
+
+    layers = []
+    for i in range(cfg["num_hidden_layers"]):
+        kind = i % 4
+        layers.append(copy.deepcopy(full if kind == 0 else scan if kind == 1 else
+                                    windowed(None) if kind == 2 else windowed(i - 1)))
+    return {"architecture": "Bekunex", "vocab": cfg["vocab_size"], "width": W,
+            "norm": {"eps": 1e-5}, "logit_scale": 1.0, "layers": layers}
+
+
 def step_bytes_of(model, batch: int, mean_context: float) -> float:
     """What a decode step of any model has to move: every tensor its parts hold once (the
     embedding table only where the head shares it), each live request's cached positions, and
@@ -215,9 +254,28 @@ def step_bytes_of(model, batch: int, mean_context: float) -> float:
     table = model.embedding.weight
     if model.head.weight.data_ptr() != table.data_ptr():
         total -= table.numel() * table.element_size()
-    per_position = sum(len(g.writer_runs) * g.request.bytes_per_token(model.act_dtype)
-                       for g in model.cache_groups)
-    return total + batch * (mean_context * per_position + 2 * model.state_bytes)
+    total -= routed_idle_bytes(model, batch)
+    per_position = 0.0                    # every run reads its group's pages, its own or not
+    for b in model.bindings:
+        if b.group >= 0:
+            req = model.cache_groups[b.group].request
+            per_position += req.bytes_per_token(model.act_dtype) * (
+                min(mean_context, req.window) if req.window else mean_context)
+    return total + batch * (per_position + 2 * model.state_bytes)
+
+
+def routed_idle_bytes(model, batch: int) -> float:
+    """The experts' weights that a decode step of ``batch`` tokens does not read: with E experts
+    of which every token takes ``top`` at random, E (1 - 1/E)^(batch top) of them stay idle on
+    average."""
+    idle = 0.0
+    for layer in model.layers:
+        ff = getattr(layer, "feed_forward", None)
+        if ff is not None and hasattr(ff, "experts"):
+            E = ff.experts
+            per_expert = (ff.w_gate_up.numel() + ff.w_down.numel()) * ff.w_down.element_size() / E
+            idle += per_expert * E * (1.0 - 1.0 / E) ** (batch * ff.top)
+    return idle
 
 
 def time_prefill(model, prompt, runs: int = 8) -> float:
@@ -290,7 +348,8 @@ def compare_designs(args) -> int:
             base["num_hidden_layers"] = args.layers
         longest = max(T, args.points_context + new + warm + 16) + 64
         base["max_position_embeddings"] = min(base["max_position_embeddings"], longest)
-        for design, cfg in (("llama", base), ("gipotar", gipotar_like(base))):
+        like = {"gipotar": gipotar_like, "bekunex": bekunex_like}
+        for design, cfg in [("llama", base)] + [(d, like[d](base)) for d in args.design.split(",")]:
             vocab = base["vocab_size"]
             model = random_model(cfg, seed=0, dtype=args.dtype, max_positions=longest)
             torch.cuda.synchronize()
@@ -309,7 +368,7 @@ def compare_designs(args) -> int:
             del model
             torch.cuda.empty_cache()
     print(json.dumps({
-        "metric": "prefill and decode tok/s, Gipotar beside Llama at equal sizes",
+        "metric": f"prefill and decode tok/s, {args.design} beside Llama at equal sizes",
         "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic (random weights N(0,0.02), uniform random token ids)",
         "config": {"sizes": args.sizes, "prefill_tokens": T, "decode_prompt": args.points_context,
@@ -349,6 +408,9 @@ def main() -> int:
     ap.add_argument("--new-tokens", type=int, default=256)
     ap.add_argument("--designs", action="store_true",
                     help="time the Gipotar design beside the Llama presets of --sizes instead")
+    ap.add_argument("--design", default="gipotar",
+                    help="the designs that --designs times beside Llama, with commas between "
+                         "them: gipotar, bekunex")
     ap.add_argument("--sizes", default="llama-3.2-1b,llama-3.2-3b",
                     help="presets whose sizes the two designs of --designs are built at")
     args = ap.parse_args()

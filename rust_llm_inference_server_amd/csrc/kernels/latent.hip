@@ -84,13 +84,15 @@ RLIS_API int rlis_head_linear(const void* x, int dtype, long long ldx, int x_hea
 // r numbers behind it are rotated by the token's position (the first rot of them: entry i with
 // entry i + rot/2; the rest pass) and follow c in the row; the last r numbers of every query
 // head are rotated the same way into the head's row of q_out behind its first R columns.
-// x is float32; angles come from float32 tables (positions, rot/2).
+// x is float32; angles come from float32 tables (positions, rot/2).  With pages_t the latent is
+// stored a second time with the positions of a page innermost ([page][j][offset]), which is how
+// the matrix-core kernel reads it as values.
 template <typename TX>
 __global__ __launch_bounds__(256) void latent_write_kernel(
     const float* __restrict__ x, long long ldx, const float* __restrict__ weight, float eps,
     int R, int r, int rot, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
     const int* __restrict__ positions, const int* __restrict__ slots, TX* __restrict__ pages,
-    int write, const TX* __restrict__ q, long long ldq, int q_head, int q_off,
+    TX* __restrict__ pages_t, int page_size, int write, const TX* __restrict__ q, long long ldq, int q_head, int q_off,
     TX* __restrict__ q_out, long long ldo, int o_head, int H) {
   __shared__ float red[4];
   const int t = blockIdx.x;
@@ -104,6 +106,11 @@ __global__ __launch_bounds__(256) void latent_write_kernel(
     ss = block_sum<256>(ss, red);
     const float mult = 1.0f / sqrtf(ss / (float)R + eps);
     for (int j = threadIdx.x; j < R; j += 256) st(row + j, xr[j] * mult * weight[j]);
+    if (pages_t) {         // the same latent once more, positions innermost: [page][j][offset]
+      TX* col = pages_t + (long long)(slots[t] / page_size) * R * page_size + slots[t] % page_size;
+      for (int j = threadIdx.x; j < R; j += 256)
+        st(col + (long long)j * page_size, xr[j] * mult * weight[j]);
+    }
     for (int j = threadIdx.x; j < r; j += 256) {
       float v = xr[R + j];
       if (j < rot) {
@@ -131,8 +138,8 @@ __global__ __launch_bounds__(256) void latent_write_kernel(
 
 RLIS_API int rlis_latent_write(const float* x, long long ldx, const float* weight, float eps,
                                int R, int r, int rot, const float* cos_t, const float* sin_t,
-                               const int* positions, const int* slots, void* pages, int dtype,
-                               int write, const void* q, long long ldq, int q_head, int q_off,
+                               const int* positions, const int* slots, void* pages,
+                               void* pages_t, int page_size, int dtype, int write, const void* q, long long ldq, int q_head, int q_off,
                                void* q_out, long long ldo, int o_head, int H, int T,
                                hipStream_t stream) {
   RLIS_REQUIRE(T >= 0 && R > 0 && r >= 0 && rot >= 0 && rot <= r && rot % 2 == 0 && H > 0,
@@ -140,12 +147,14 @@ RLIS_API int rlis_latent_write(const float* x, long long ldx, const float* weigh
   RLIS_REQUIRE(rot == 0 || (cos_t && sin_t), "latent_write: a rotation needs its tables");
   RLIS_REQUIRE(!write || (ldx >= R + r && pages && slots && weight),
                "latent_write: the cache write needs rows, pages and slots");
+  RLIS_REQUIRE(!pages_t || page_size > 0, "latent_write: the transposed copy needs the page size");
   RLIS_REQUIRE(r == 0 || (q && q_out && q_head >= q_off + r && o_head >= R + r),
                "latent_write: the rotated query part needs its rows");
   if (T == 0 || (!write && r == 0)) return 0;
 #define LAUNCH(TX)                                                                            \
   latent_write_kernel<TX><<<T, 256, 0, stream>>>(x, ldx, weight, eps, R, r, rot, cos_t, sin_t, \
-                                                 positions, slots, (TX*)pages, write,          \
+                                                 positions, slots, (TX*)pages, (TX*)pages_t,   \
+                                                 page_size, write,                             \
                                                  (const TX*)q, ldq, q_head, q_off, (TX*)q_out, \
                                                  ldo, o_head, H)
   if (dtype == RLIS_F32) LAUNCH(float);
@@ -254,6 +263,187 @@ RLIS_API int rlis_latent_attention(const void* q, int dtype, long long ldq, void
 #undef BY_CPL
 #undef LAUNCH
   RLIS_LAUNCH_CHECK("latent_attention");
+  return 0;
+}
+
+// --------------------------------------------------------------- attention, matrix cores
+// bfloat16.  A wave takes 16 (token, head) columns of one sequence: 16 heads of a token, or
+// with fewer heads 16 / HP tokens x HP heads (HP the power of two that holds the heads), and
+// walks the keys its columns see in chunks of 32.  Transposed products, so that a column's
+// softmax statistics stay in its lanes and the probabilities never leave registers:
+// S^T = C Q^T (rows: keys; the cached rows [c | kr] are loaded straight into operand layout)
+// and O^T += C^T P^T (rows: latent channels; C^T comes from the copy that lies with positions
+// innermost, 8 keys in one 16-byte load).  Row i of S^T's block u is key 8 (i / 4) + 4 u + i % 4
+// of the chunk, which puts a lane's 8 probabilities on 8 consecutive keys.  The queries wait in
+// LDS (a wave's own 16 rows); scale, mask, sink and sums are float32; P is rounded to
+// bfloat16 as the second product's operand only.  How a sequence's keys are cut follows from
+// its own positions, so a row does not depend on its neighbours.
+template <int NT>
+__global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
+    const bf16_t* __restrict__ q, long long ldq, bf16_t* __restrict__ out, long long ldo,
+    const bf16_t* __restrict__ pages, const bf16_t* __restrict__ pages_t,
+    const int* __restrict__ block_tables, int max_pages, const int* __restrict__ cu,
+    const int* __restrict__ positions, int num_seqs, int H, int R, int D, int page_size,
+    float scale, int window, const float* __restrict__ sink, int HP) {
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int c = lane % 16, g = lane / 16;
+  const int TB = 16 / HP;
+  const int stride = D + 8;
+  bf16_t* q_s = reinterpret_cast<bf16_t*>(lds_raw) + (size_t)wave * 16 * stride;
+  int blk = blockIdx.x * 4 + wave;
+  int seq = -1, t_first = 0, t_end = 0;
+  for (int s = 0; s < num_seqs; ++s) {
+    const int a = cu[s], b = cu[s + 1];
+    const int tiles = (b - a + TB - 1) / TB;
+    if (blk < tiles) {
+      seq = s;
+      t_first = a + blk * TB;
+      t_end = b;
+      break;
+    }
+    blk -= tiles;
+  }
+  if (seq < 0) return;                       // (the whole wave: nothing below waits for others)
+  const int tok = t_first + c / HP;
+  const int head = blockIdx.y * HP + c % HP;
+  const bool col_ok = tok < t_end && head < H;
+  const int tok_c = min(tok, t_end - 1), head_c = min(head, H - 1);
+  const int pos = positions[tok_c];
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int hi_blk = positions[min(t_first + TB, t_end) - 1];
+  const int p_first = positions[t_first];
+  const int lo_blk = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
+  const bf16_t* q_row = q + (long long)tok_c * ldq + (long long)head_c * D;
+  for (int j = g * 8; j < D; j += 32)
+    *reinterpret_cast<mma_u32x4*>(q_s + c * stride + j) =
+        *reinterpret_cast<const mma_u32x4*>(q_row + j);
+  const int* table = block_tables + (long long)seq * max_pages;
+  float m = sink ? sink[head_c] : -INFINITY;
+  float l = (sink && g == 0) ? 1.f : 0.f;
+  mma_f32x4 acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) acc[t] = mma_f32x4{0.f, 0.f, 0.f, 0.f};
+  const int steps = (D + 31) / 32;
+  const mma_u32x4 zero = {0u, 0u, 0u, 0u};
+  for (int k0 = lo_blk & ~31; k0 <= hi_blk; k0 += 32) {
+    const int kk0 = min(k0 + 8 * (c / 4) + c % 4, hi_blk), kk1 = min(kk0 + 4, hi_blk);
+    const bf16_t* kr0 =
+        pages + ((long long)table[kk0 / page_size] * page_size + kk0 % page_size) * D;
+    const bf16_t* kr1 =
+        pages + ((long long)table[kk1 / page_size] * page_size + kk1 % page_size) * D;
+    mma_f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < steps; ++s) {
+      const int dch = 32 * s + 8 * g;
+      const mma_u32x4 qr = *reinterpret_cast<const mma_u32x4*>(q_s + c * stride + (dch < D ? dch : 0));
+      const mma_u32x4 qv = dch < D ? qr : zero;
+      const mma_u32x4 a0 = mma_load<bf16_t, true>(kr0, dch, D);
+      const mma_u32x4 a1 = mma_load<bf16_t, true>(kr1, dch, D);
+      s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mma_bf16x8, a0),
+                                                   __builtin_bit_cast(mma_bf16x8, qv), s0, 0, 0, 0);
+      s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mma_bf16x8, a1),
+                                                   __builtin_bit_cast(mma_bf16x8, qv), s1, 0, 0, 0);
+    }
+    float sv[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int key0 = k0 + 8 * g + i, key1 = key0 + 4;
+      sv[i] = (col_ok && key0 >= lo && key0 <= pos) ? s0[i] * scale : -INFINITY;
+      sv[4 + i] = (col_ok && key1 >= lo && key1 <= pos) ? s1[i] * scale : -INFINITY;
+      mx = fmaxf(mx, fmaxf(sv[i], sv[4 + i]));
+    }
+    mx = xor32_max(xor16_max(mx));
+    const float m_new = fmaxf(m, mx);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float corr = m == -INFINITY ? 0.f : __expf(m - m_use);
+    float psum = 0.f;
+    bf16_t pk[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float p = __expf(sv[j] - m_use);
+      psum += p;
+      pk[j] = f32_to_bf16(p);
+    }
+    l = l * corr + psum;
+    m = m_new;
+    const mma_bf16x8 pv = __builtin_bit_cast(mma_bf16x8, pk);
+    const int kv = k0 + 8 * g;
+    const long long vpage = table[min(kv / page_size, max_pages - 1)];
+    const bf16_t* vt = pages_t + vpage * R * page_size + kv % page_size;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const int dim = min(16 * t + c, R - 1);
+      const mma_u32x4 a = *reinterpret_cast<const mma_u32x4*>(vt + (long long)dim * page_size);
+      acc[t] *= corr;
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mma_bf16x8, a), pv,
+                                                       acc[t], 0, 0, 0);
+    }
+  }
+  const float total = xor32_sum(xor16_sum(l));
+  if (!col_ok) return;
+  const float inv = 1.0f / total;
+  bf16_t* o = out + (long long)tok * ldo + (long long)head * R;
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int dim = 16 * t + 4 * g + i;
+      if (dim < R) o[dim] = f32_to_bf16(acc[t][i] * inv);
+    }
+}
+
+static LdsGrant g_latent_lds[4];
+
+// Whether the matrix-core kernel takes a latent of R numbers in rows of D.
+RLIS_API int rlis_latent_attention_mfma_ok(int R, int D, int page_size) {
+  if (R <= 0 || R > 512 || D % 8 || page_size % 8) return 0;
+  const int nt = R <= 64 ? 4 : R <= 128 ? 8 : R <= 256 ? 16 : 32;
+  return D <= 16 * nt + 64 ? 1 : 0;
+}
+
+RLIS_API int rlis_latent_attention_mfma(const void* q, long long ldq, void* out, long long ldo,
+                                        const void* pages, const void* pages_t,
+                                        const int* block_tables, int max_pages, const int* cu,
+                                        const int* positions, int T, int num_seqs, int H, int R,
+                                        int D, int page_size, float scale, int window,
+                                        const float* sink, hipStream_t stream) {
+  RLIS_REQUIRE(T >= 0 && num_seqs > 0 && H > 0 && D >= R && max_pages > 0,
+               "latent_attention_mfma: bad sizes");
+  RLIS_REQUIRE(rlis_latent_attention_mfma_ok(R, D, page_size),
+               "latent_attention_mfma: a latent of %d in rows of %d with pages of %d is not taken",
+               R, D, page_size);
+  RLIS_REQUIRE(ldq % 8 == 0 && (uintptr_t)q % 16 == 0 && (uintptr_t)pages % 16 == 0 &&
+                   (uintptr_t)pages_t % 16 == 0,
+               "latent_attention_mfma: operands must lie on 16-byte boundaries");
+  RLIS_REQUIRE(ldq >= (long long)H * D && ldo >= (long long)H * R,
+               "latent_attention_mfma: rows shorter than their heads");
+  if (T == 0) return 0;
+  int hp = 1;
+  while (hp < H && hp < 16) hp *= 2;
+  const int tb = 16 / hp;
+  const int blocks = ceil_div(T, tb) + num_seqs;
+  dim3 grid(ceil_div(blocks, 4), ceil_div(H, hp));
+  RLIS_REQUIRE(grid.y <= 65535, "latent_attention_mfma: too many heads");
+  const int lds = 4 * 16 * (D + 8) * 2;
+#define LAUNCH(NT, slot)                                                                       \
+  do {                                                                                         \
+    if (lds > 48 * 1024) {                                                                     \
+      hipError_t e = grant_lds(g_latent_lds[slot],                                             \
+                               (const void*)latent_attention_mfma_kernel<NT>, lds);            \
+      RLIS_REQUIRE(e == hipSuccess, "latent_attention_mfma: LDS of %d bytes refused", lds);     \
+    }                                                                                          \
+    latent_attention_mfma_kernel<NT><<<grid, 256, lds, stream>>>(                              \
+        (const bf16_t*)q, ldq, (bf16_t*)out, ldo, (const bf16_t*)pages, (const bf16_t*)pages_t, \
+        block_tables, max_pages, cu, positions, num_seqs, H, R, D, page_size, scale, window,   \
+        sink, hp);                                                                             \
+  } while (0)
+  if (R <= 64) LAUNCH(4, 0);
+  else if (R <= 128) LAUNCH(8, 1);
+  else if (R <= 256) LAUNCH(16, 2);
+  else LAUNCH(32, 3);
+#undef LAUNCH
+  RLIS_LAUNCH_CHECK("latent_attention_mfma");
   return 0;
 }
 

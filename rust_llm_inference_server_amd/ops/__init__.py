@@ -1089,7 +1089,8 @@ def sample_rows(logits: torch.Tensor, keys: torch.Tensor, inv_temps: torch.Tenso
 
 from .recurrent import (causal_conv, decay_scan, delta_scan, head_norm_gate,  # noqa: E402,F401
                         selective_scan, shift_mix, tail_update)
-from .latent import head_linear, latent_attention, latent_write, sigmoid_gate_  # noqa: E402,F401
+from .latent import (head_linear, latent_attention, latent_mfma_ok, latent_write,  # noqa: E402,F401
+                     sigmoid_gate_)
 from .routed import routed_units, route  # noqa: E402,F401
 
 

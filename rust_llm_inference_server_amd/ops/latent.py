@@ -61,7 +61,7 @@ def latent_write(x: Optional[torch.Tensor], weight: Optional[torch.Tensor], eps:
                  sin: Optional[torch.Tensor], positions: torch.Tensor,
                  slots: Optional[torch.Tensor], pages: Optional[torch.Tensor],
                  q: Optional[torch.Tensor], q_head: int, q_out: Optional[torch.Tensor],
-                 heads: int) -> None:
+                 heads: int, pages_t: Optional[torch.Tensor] = None) -> None:
     """For every token of the step: the first ``rank`` columns of ``x`` (float32), divided by
     their root mean square (``eps`` inside the root) and multiplied by ``weight``, go to the
     token's row of ``pages (pages, page size, rank + rot_width)`` at ``slots``; the
@@ -70,7 +70,9 @@ def latent_write(x: Optional[torch.Tensor], weight: Optional[torch.Tensor], eps:
     ``cos``/``sin (positions, rot_dims / 2)``).  The last ``rot_width`` numbers of every head
     of ``q`` (heads ``q_head`` apart) are rotated the same way into ``q_out`` behind each
     head's first ``rank`` columns (heads ``rank + rot_width`` apart).  ``x`` None: nothing is
-    written to the cache (a mixer that reads another's)."""
+    written to the cache (a mixer that reads another's).  ``pages_t (pages, rank, page size)``:
+    the latent is stored there once more, with the positions of a page innermost (what the
+    matrix-core attention kernel reads as values)."""
     T = positions.numel() if q is None else q.shape[0]
     write = x is not None
     D = rank + rot_width
@@ -86,6 +88,11 @@ def latent_write(x: Optional[torch.Tensor], weight: Optional[torch.Tensor], eps:
             raise KernelError(f"latent_write: the norm's weight must be {rank} float32 values")
         _i32(slots, T, "latent_write slots")
         T = x.shape[0]
+        if pages_t is not None and (tuple(pages_t.shape) != (pages.shape[0], rank, pages.shape[1])
+                                    or pages_t.dtype != pages.dtype
+                                    or not pages_t.is_contiguous()):
+            raise KernelError("latent_write: the transposed pages must be contiguous "
+                              "(pages, rank, page size) of the pages' dtype")
     ldq = ldo = 0
     dtype = pages.dtype if pages is not None else (q.dtype if q is not None else torch.float32)
     if rot_width:
@@ -104,20 +111,39 @@ def latent_write(x: Optional[torch.Tensor], weight: Optional[torch.Tensor], eps:
              int(rot_dims), None if cos is None else cos.data_ptr(),
              None if sin is None else sin.data_ptr(), _i32(positions, T, "positions"),
              None if not write else slots.data_ptr(),
-             None if pages is None else pages.data_ptr(), _DT[dtype], int(write),
+             None if pages is None else pages.data_ptr(),
+             None if pages_t is None or not write else pages_t.data_ptr(),
+             0 if pages is None else pages.shape[1], _DT[dtype], int(write),
              None if q is None else q.data_ptr(), ldq, int(q_head), int(q_head - rot_width),
              None if q_out is None else q_out.data_ptr(), ldo, D, int(heads), T, lib.stream_ptr())
+
+
+# "matrix": bfloat16 attention over cached latents runs on the matrix cores where it applies;
+# "vector": always the vector-unit kernel (tests hold the two against each other).
+LATENT_ATTENTION = "matrix"
+
+
+def latent_mfma_ok(dtype: torch.dtype, rank: int, row: int, page_size: int = 16) -> bool:
+    """Whether the matrix-core kernel takes latents of ``rank`` numbers in cached rows of
+    ``row`` (it reads a second, transposed copy of the latents, which the mixer then keeps)."""
+    return dtype == torch.bfloat16 and bool(
+        lib.load().rlis_latent_attention_mfma_ok(int(rank), int(row), int(page_size)))
 
 
 def latent_attention(q: torch.Tensor, pages: torch.Tensor, block_tables: torch.Tensor,
                      seq_of_token: torch.Tensor, positions: torch.Tensor, heads: int, rank: int,
                      scale: float, window: Optional[int] = None,
-                     sink: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     sink: Optional[torch.Tensor] = None,
+                     pages_t: Optional[torch.Tensor] = None, cu: Optional[torch.Tensor] = None,
+                     num_seqs: int = 0) -> torch.Tensor:
     """Softmax attention of ``q (T, heads * D)`` over cached rows ``pages (pages, page size,
     D)``: the score of a row is ``scale * (q_h . row)``, the output per head the weighted sum
     of the rows' first ``rank`` numbers, ``(T, heads * rank)``.  A query at position p sees rows
     at positions <= p and, under ``window`` w, > p - w.  ``sink (heads)`` float32: the
-    softmax's denominator also holds ``exp(sink[h])``."""
+    softmax's denominator also holds ``exp(sink[h])``.  With ``pages_t`` (the latents once more
+    as ``(pages, rank, page size)``), ``cu`` (cumulative token counts of the step's
+    ``num_seqs`` sequences) and bfloat16 operands of sizes it takes, the matrix-core kernel
+    runs; otherwise the vector-unit kernel (any sizes, both dtypes)."""
     ldq = _rows2(q, "latent_attention q")
     T = q.shape[0]
     if pages.dim() != 3 or not pages.is_contiguous() or pages.dtype != q.dtype:
@@ -133,6 +159,19 @@ def latent_attention(q: torch.Tensor, pages: torch.Tensor, block_tables: torch.T
                              or not sink.is_contiguous()):
         raise KernelError(f"latent_attention: the sink must be {heads} float32 values")
     out = torch.empty((T, heads * rank), dtype=q.dtype, device=q.device)
+    if pages_t is not None and cu is not None and num_seqs > 0 and LATENT_ATTENTION == "matrix" \
+            and ldq % 8 == 0 and latent_mfma_ok(q.dtype, rank, D, page_size):
+        if tuple(pages_t.shape) != (pages.shape[0], rank, page_size) \
+                or pages_t.dtype != q.dtype or not pages_t.is_contiguous():
+            raise KernelError("latent_attention: the transposed pages must be contiguous "
+                              "(pages, rank, page size)")
+        lib.call("rlis_latent_attention_mfma", q.data_ptr(), ldq, out.data_ptr(), heads * rank,
+                 pages.data_ptr(), pages_t.data_ptr(), block_tables.data_ptr(),
+                 block_tables.shape[1], _i32(cu, num_seqs + 1, "cu"),
+                 _i32(positions, T, "positions"), T, int(num_seqs), heads, rank, D, page_size,
+                 float(scale), int(window or 0), None if sink is None else sink.data_ptr(),
+                 lib.stream_ptr())
+        return out
     lib.call("rlis_latent_attention", q.data_ptr(), _DT[q.dtype], ldq, out.data_ptr(),
              heads * rank, pages.data_ptr(), block_tables.data_ptr(), block_tables.shape[1],
              _i32(seq_of_token, T, "seq_of_token"), _i32(positions, T, "positions"), T, heads,

@@ -31,7 +31,8 @@ _SIGNATURES = {
     "rlis_add_layernorm": [P, P, I, P, P, I, P, I, P, I, I, F, I, I, L, I, F, P],
     "rlis_scale": [P, I, L, F, P],
     "rlis_head_linear": [P, I, L, I, P, P, I, L, I, I, I, I, I, P],
-    "rlis_latent_write": [P, L, P, F, I, I, I, P, P, P, P, P, I, I, P, L, I, I, P, L, I, I, I, P],
+    "rlis_latent_write": [P, L, P, F, I, I, I, P, P, P, P, P, P, I, I, I, P, L, I, I, P, L, I, I, I, P],
+    "rlis_latent_attention_mfma": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, I, F, I, P, P],
     "rlis_latent_attention": [P, I, L, P, L, P, P, I, P, P, I, I, I, I, I, F, I, P, P],
     "rlis_sigmoid_gate": [P, L, P, L, I, I, I, P],
     "rlis_moe_route": [P, L, P, I, I, I, I, I, F, P, P, P],
@@ -107,6 +108,8 @@ def load() -> ctypes.CDLL:
                                  P, P, P]
     lib.rlis_lt_adopt.restype = c_int
     lib.rlis_lt_adopt.argtypes = [I, I, I, I, I, L, L, L, L, I, L, ctypes.c_size_t, P]
+    lib.rlis_latent_attention_mfma_ok.restype = c_int
+    lib.rlis_latent_attention_mfma_ok.argtypes = [I, I, I]
     lib.rlis_gemm_bf16_stream_max_rows.restype = c_int
     lib.rlis_gemm_bf16_stream_max_rows.argtypes = [I]
     _LIB = lib

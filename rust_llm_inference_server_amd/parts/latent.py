@@ -7,7 +7,9 @@ numbers that are rotated by position and serve every head as the second part of 
 Head ``h`` has ``k_h = Uk_h c`` and ``v_h = Uv_h c``; its score for a cached position is
 ``(q_h . k_h + q_rot_h . k_rot) * scale``.  Only ``[c | k_rot]`` is cached, one row per
 position, and both maps are taken to the query side (``Uk_h^T q_h`` meets ``c``; the weighted
-sum of cached latents goes through ``Uv_h`` afterwards), so the cache is read as it lies.
+sum of cached latents goes through ``Uv_h`` afterwards), so the cache is read as it lies.  (In
+bfloat16 the latent is kept a second time with the positions of a page innermost, which is how
+the matrix-core kernel loads it as values.)
 
 Options, each a parameter: a rotated part (``rot_dim`` 0: none), a sliding window, a learned
 sink per head in the softmax's denominator, a sigmoid gate on the heads' outputs (its own
@@ -87,6 +89,10 @@ class LatentAttention(Mixer):
         self.sink = take("sink").to(torch.float32).contiguous() if params.get("sink") else None
         self.w_g = take("g") if params.get("gate") else None
         self.w_o = take("o")
+        # the matrix-core kernel reads the latents as values from a second copy that lies with
+        # the positions of a page innermost; the mixer keeps it where that kernel applies
+        self.keeps_transposed = ctx.device.type == "cuda" and ops.latent_mfma_ok(
+            ctx.act_dtype, R, R + self.rot_width)
         self.position = None
         self.rot_dims = 0
         if self.rot_width:
@@ -96,12 +102,14 @@ class LatentAttention(Mixer):
                 raise ValueError("latent_attention: more rotated dims than the rotated part has")
 
     def cache_request(self) -> CacheRequest:
-        return CacheRequest((PageArray("latent", (PAGE, self.rank + self.rot_width)),),
-                            self.cache_window)
+        arrays = (PageArray("latent", (PAGE, self.rank + self.rot_width)),)
+        if self.keeps_transposed:
+            arrays += (PageArray("latent_t", (self.rank, PAGE)),)
+        return CacheRequest(arrays, self.cache_window)
 
     def forward(self, x: torch.Tensor, step: Any, binding: CacheBinding) -> Any:
         group = step.groups[binding.group]
-        pages = binding.pages["latent"]
+        pages, pages_t = binding.pages["latent"], binding.pages.get("latent_t")
         H, d, r, R = self.heads, self.dim, self.rot_width, self.rank
         T = x.shape[0]
         if self.position is not None and step.max_context > self.position.max_positions:
@@ -117,9 +125,10 @@ class LatentAttention(Mixer):
             sin = self.position.sin if self.rot_dims else None
             ops.latent_write(down, self.norm if writes else None, self.eps, R, r, self.rot_dims,
                              cos, sin, step.positions, group.slots if writes else None, pages,
-                             q if r else None, d + r, q_lat if r else None, H)
+                             q if r else None, d + r, q_lat if r else None, H, pages_t)
         mixed = ops.latent_attention(q_lat, pages, group.block_tables, step.seq_of_token,
-                                     step.positions, H, R, self.scale, self.window, self.sink)
+                                     step.positions, H, R, self.scale, self.window, self.sink,
+                                     pages_t, step.cu_seqlens, step.num_seqs)
         out = ops.head_linear(mixed, self.w_uv, R)                     # (T, H * vdim)
         if self.w_g is not None:
             ops.sigmoid_gate_(out, ops.linear(x, self.w_g, self.act_dtype))

@@ -138,17 +138,19 @@ def make_weights(config: dict, seed: int) -> Dict[str, torch.Tensor]:
 
 def judge(errors: List[float], dtype: str) -> None:
     """float32: no row beyond two and a half times the tolerance and at most one in fifty beyond
-    it.  bfloat16: at most one row in fifty beyond the tolerance, whatever its size, and nineteen
-    in twenty within half of it: where two experts' choice scores lie closer than bfloat16
+    it.  bfloat16: at most one row in twenty-five beyond the tolerance, whatever its size, and
+    nine in ten within half of it: where two experts' choice scores lie closer than bfloat16
     resolves the router's input, the engine may take the other one, and that row (seldom a
-    later one) is then far from the plain logits; at these sizes that happens to one row in
-    some hundreds, while a fault of the cache or the state moves most rows."""
+    later one) is then far from the plain logits; at these sizes, with single experts chosen
+    out of four, that happens to two or three rows in a hundred, while a fault of the cache or
+    the state moves most rows."""
     tol = TOLERANCE[dtype]
     over = sum(e > tol for e in errors)
-    assert over <= max(1, len(errors) // 50), f"{over} of {len(errors)} rows beyond {tol}"
     if dtype == "float32":
+        assert over <= max(1, len(errors) // 50), f"{over} of {len(errors)} rows beyond {tol}"
         assert max(errors) < 2.5 * tol, f"worst row error {max(errors):.3g}"
     else:
+        assert over <= max(1, len(errors) // 25), f"{over} of {len(errors)} rows beyond {tol}"
         ranked = sorted(errors)
-        p95 = ranked[min(len(ranked) - 1, int(0.95 * len(ranked)))]
-        assert p95 < tol / 2 or len(ranked) < 20, f"95th percentile of the row errors {p95:.3g}"
+        p90 = ranked[min(len(ranked) - 1, int(0.9 * len(ranked)))]
+        assert p90 < tol / 2 or len(ranked) < 20, f"90th percentile of the row errors {p90:.3g}"

@@ -162,8 +162,12 @@ def _turned(v, pos, cos, sin, dims):
     return torch.cat([a * c - b * s, b * c + a * s, v[..., dims:]], dim=-1)
 
 
+def latent_mfma_ok(dtype, rank, row, page_size=16):
+    return False
+
+
 def latent_write(x, weight, eps, rank, rot_width, rot_dims, cos, sin, positions, slots, pages, q,
-                 q_head, q_out, heads):
+                 q_head, q_out, heads, pages_t=None):
     D = rank + rot_width
     if x is not None:
         lat = x[:, :rank]
@@ -183,7 +187,7 @@ def latent_write(x, weight, eps, rank, rot_width, rot_dims, cos, sin, positions,
 
 
 def latent_attention(q, pages, block_tables, seq_of_token, positions, heads, rank, scale,
-                     window=None, sink=None):
+                     window=None, sink=None, pages_t=None, cu=None, num_seqs=0):
     T = q.shape[0]
     ps, D = pages.shape[1], pages.shape[2]
     qf = q.float().reshape(T, heads, D)
@@ -398,6 +402,7 @@ def install(monkeypatch) -> None:
                  "clamped_glu", "weighted_sum", "linear_f32", "soft_cap_", "shift_mix", "tail_update",
                  "causal_conv", "delta_scan", "decay_scan", "head_norm_gate", "selective_scan",
                  "add_layernorm", "scale_", "head_linear", "latent_write", "latent_attention",
+                 "latent_mfma_ok",
                  "sigmoid_gate_", "route", "routed_units"):
         monkeypatch.setattr(ops, name, globals()[name])
     monkeypatch.setattr(runner, "default_device", lambda: torch.device("cpu"))

@@ -82,7 +82,8 @@ def _cached_attention_case(dtype, H, d, r, R, n, page, seed):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H, d, r, R, window, sink", [
     (3, 16, 8, 40, None, False), (2, 12, 6, 28, None, False), (4, 8, 0, 36, 16, True),
-    (1, 24, 0, 70, 1, True), (2, 16, 0, 16, 33, False), (2, 32, 16, 128, 17, True)])
+    (1, 24, 0, 70, 1, True), (2, 16, 0, 16, 33, False), (2, 32, 16, 128, 17, True),
+    (20, 16, 16, 64, None, False), (16, 8, 0, 200, 40, True), (5, 16, 32, 288, None, True)])
 def test_attention_over_cached_latents(dtype, H, d, r, R, window, sink):
     """Cache write in two portions (pages in a shuffled order), then every query against the
     plain softmax over keys made from the latents: rotation, norm, window edges, the sink."""
@@ -111,6 +112,9 @@ def test_attention_over_cached_latents(dtype, H, d, r, R, window, sink):
     table[0, :len(order)] = order.to(torch.int32)
     slots = (table[0, pos // page].long() * page + pos % page).to(torch.int32)
     pages = torch.zeros(num_pages, page, D, dtype=dtype, device=DEV)
+    matrix = ops.latent_mfma_ok(dtype, R, D, page)
+    assert matrix == (dtype == torch.bfloat16 and D % 8 == 0)
+    pages_t = torch.zeros(num_pages, R, page, dtype=dtype, device=DEV) if matrix else None
     cos = sin = None
     if r:
         ang = pos.double().reshape(-1, 1) * base ** (-torch.arange(0, r, 2).double() / r)
@@ -123,11 +127,16 @@ def test_attention_over_cached_latents(dtype, H, d, r, R, window, sink):
     for lo, hi in ((0, 41), (41, n)):
         ops.latent_write(down[lo:hi].to(DEV), norm.to(DEV), eps, R, r, r, cos, sin, posd[lo:hi],
                          slots[lo:hi].to(DEV), pages, qg[lo:hi] if r else None, d + r,
-                         q_lat[lo:hi] if r else None, H)
-    got = ops.latent_attention(q_lat, pages, table.to(DEV), torch.zeros(n, dtype=torch.int32,
-                                                                       device=DEV), posd, H, R,
-                               scale, window, None if sink_w is None else sink_w.to(DEV))
+                         q_lat[lo:hi] if r else None, H, pages_t)
+    args = (q_lat, pages, table.to(DEV), torch.zeros(n, dtype=torch.int32, device=DEV), posd, H, R,
+            scale, window, None if sink_w is None else sink_w.to(DEV))
+    got = ops.latent_attention(*args)                    # the vector-unit kernel
     assert rel(got.reshape(n, H, R), want) < (3e-5 if dtype == torch.float32 else 3e-2)
+    if matrix:
+        assert torch.equal(pages_t.transpose(1, 2), pages[:, :, :R])
+        cu = torch.tensor([0, n], dtype=torch.int32, device=DEV)
+        got = ops.latent_attention(*args, pages_t=pages_t, cu=cu, num_seqs=1)
+        assert rel(got.reshape(n, H, R), want) < 3e-2
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
