@@ -278,7 +278,7 @@ RLIS_API int rlis_latent_attention(const void* q, int dtype, long long ldq, void
 // LDS (a wave's own 16 rows); scale, mask, sink and sums are float32; P is rounded to
 // bfloat16 as the second product's operand only.  How a sequence's keys are cut follows from
 // its own positions, so a row does not depend on its neighbours.
-template <int NT>
+template <int NT, bool SPLIT>
 __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     const bf16_t* __restrict__ q, long long ldq, bf16_t* __restrict__ out, long long ldo,
     const bf16_t* __restrict__ pages, const bf16_t* __restrict__ pages_t,
@@ -290,8 +290,10 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
   const int c = lane % 16, g = lane / 16;
   const int TB = 16 / HP;
   const int stride = D + 8;
-  bf16_t* q_s = reinterpret_cast<bf16_t*>(lds_raw) + (size_t)wave * 16 * stride;
-  int blk = blockIdx.x * 4 + wave;
+  // SPLIT: the four waves share one block of columns and take every fourth chunk of keys each
+  // (steps of few tokens: the grid is small and a context is a long walk for one wave)
+  bf16_t* q_s = reinterpret_cast<bf16_t*>(lds_raw) + (SPLIT ? 0 : (size_t)wave * 16 * stride);
+  int blk = SPLIT ? blockIdx.x : blockIdx.x * 4 + wave;
   int seq = -1, t_first = 0, t_end = 0;
   for (int s = 0; s < num_seqs; ++s) {
     const int a = cu[s], b = cu[s + 1];
@@ -304,7 +306,7 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     }
     blk -= tiles;
   }
-  if (seq < 0) return;                       // (the whole wave: nothing below waits for others)
+  if (seq < 0) return;       // (the whole wave, and with SPLIT the whole workgroup)
   const int tok = t_first + c / HP;
   const int head = blockIdx.y * HP + c % HP;
   const bool col_ok = tok < t_end && head < H;
@@ -315,34 +317,47 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
   const int p_first = positions[t_first];
   const int lo_blk = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
   const bf16_t* q_row = q + (long long)tok_c * ldq + (long long)head_c * D;
-  for (int j = g * 8; j < D; j += 32)
-    *reinterpret_cast<mma_u32x4*>(q_s + c * stride + j) =
-        *reinterpret_cast<const mma_u32x4*>(q_row + j);
+  if (!SPLIT || wave == 0)
+    for (int j = g * 8; j < D; j += 32)
+      *reinterpret_cast<mma_u32x4*>(q_s + c * stride + j) =
+          *reinterpret_cast<const mma_u32x4*>(q_row + j);
+  if (SPLIT) __syncthreads();
   const int* table = block_tables + (long long)seq * max_pages;
-  float m = sink ? sink[head_c] : -INFINITY;
-  float l = (sink && g == 0) ? 1.f : 0.f;
+  const bool opens = !SPLIT || wave == 0;        // whose sums the sink opens
+  float m = (sink && opens) ? sink[head_c] : -INFINITY;
+  float l = (sink && opens && g == 0) ? 1.f : 0.f;
   mma_f32x4 acc[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) acc[t] = mma_f32x4{0.f, 0.f, 0.f, 0.f};
   const int steps = (D + 31) / 32;
   const mma_u32x4 zero = {0u, 0u, 0u, 0u};
-  for (int k0 = lo_blk & ~31; k0 <= hi_blk; k0 += 32) {
+  constexpr int GS = NT >= 32 ? 4 : NT == 4 ? 4 : 6;     // key loads asked for together
+  for (int k0 = (lo_blk & ~31) + (SPLIT ? 32 * wave : 0); k0 <= hi_blk;
+       k0 += SPLIT ? 128 : 32) {
     const int kk0 = min(k0 + 8 * (c / 4) + c % 4, hi_blk), kk1 = min(kk0 + 4, hi_blk);
     const bf16_t* kr0 =
         pages + ((long long)table[kk0 / page_size] * page_size + kk0 % page_size) * D;
     const bf16_t* kr1 =
         pages + ((long long)table[kk1 / page_size] * page_size + kk1 % page_size) * D;
     mma_f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
-    for (int s = 0; s < steps; ++s) {
-      const int dch = 32 * s + 8 * g;
-      const mma_u32x4 qr = *reinterpret_cast<const mma_u32x4*>(q_s + c * stride + (dch < D ? dch : 0));
-      const mma_u32x4 qv = dch < D ? qr : zero;
-      const mma_u32x4 a0 = mma_load<bf16_t, true>(kr0, dch, D);
-      const mma_u32x4 a1 = mma_load<bf16_t, true>(kr1, dch, D);
-      s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mma_bf16x8, a0),
-                                                   __builtin_bit_cast(mma_bf16x8, qv), s0, 0, 0, 0);
-      s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mma_bf16x8, a1),
-                                                   __builtin_bit_cast(mma_bf16x8, qv), s1, 0, 0, 0);
+    for (int sb = 0; sb < steps; sb += GS) {
+      mma_u32x4 a0[GS], a1[GS];
+#pragma unroll
+      for (int u = 0; u < GS; ++u) {      // (past the row's end: a clamped address and zeros)
+        a0[u] = mma_load<bf16_t, true>(kr0, 32 * (sb + u) + 8 * g, D);
+        a1[u] = mma_load<bf16_t, true>(kr1, 32 * (sb + u) + 8 * g, D);
+      }
+#pragma unroll
+      for (int u = 0; u < GS; ++u) {
+        const int dch = 32 * (sb + u) + 8 * g;
+        const mma_u32x4 qr =
+            *reinterpret_cast<const mma_u32x4*>(q_s + c * stride + (dch < D ? dch : 0));
+        const mma_bf16x8 qv = __builtin_bit_cast(mma_bf16x8, dch < D ? qr : zero);
+        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mma_bf16x8, a0[u]), qv,
+                                                     s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mma_bf16x8, a1[u]), qv,
+                                                     s1, 0, 0, 0);
+      }
     }
     float sv[8];
     float mx = -INFINITY;
@@ -380,6 +395,42 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
                                                        acc[t], 0, 0, 0);
     }
   }
+  if (SPLIT) {
+    // waves 2, 3 hand their sums to waves 0, 1, then wave 1 hands the pair's to wave 0:
+    // per lane m, l and the 4 NT sums, laid out [value][lane]
+    float* hand = reinterpret_cast<float*>(lds_raw + 16 * stride * 2) ;
+    constexpr int kVals = 4 * NT + 2;
+#pragma unroll
+    for (int round = 0; round < 2; ++round) {
+      const bool gives = round == 0 ? wave >= 2 : wave == 1;
+      const bool takes = round == 0 ? wave < 2 : wave == 0;
+      float* mine = hand + (size_t)(round == 0 ? wave & 1 : 0) * kVals * kWave + lane;
+      __syncthreads();
+      if (gives) {
+        mine[0] = m;
+        mine[kWave] = l;
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) mine[(size_t)(2 + 4 * t + i) * kWave] = acc[t][i];
+      }
+      __syncthreads();
+      if (takes) {
+        const float m_b = mine[0], l_b = mine[kWave];
+        const float m_ab = fmaxf(m, m_b);
+        const float fa = m == -INFINITY ? 0.f : __expf(m - m_ab);
+        const float fb = m_b == -INFINITY ? 0.f : __expf(m_b - m_ab);
+        l = l * fa + l_b * fb;
+        m = m_ab;
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            acc[t][i] = acc[t][i] * fa + mine[(size_t)(2 + 4 * t + i) * kWave] * fb;
+      }
+    }
+    if (wave != 0) return;
+  }
   const float total = xor32_sum(xor16_sum(l));
   if (!col_ok) return;
   const float inv = 1.0f / total;
@@ -393,7 +444,7 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     }
 }
 
-static LdsGrant g_latent_lds[4];
+static LdsGrant g_latent_lds[8];
 
 // Whether the matrix-core kernel takes a latent of R numbers in rows of D.
 RLIS_API int rlis_latent_attention_mfma_ok(int R, int D, int page_size) {
@@ -407,7 +458,8 @@ RLIS_API int rlis_latent_attention_mfma(const void* q, long long ldq, void* out,
                                         const int* block_tables, int max_pages, const int* cu,
                                         const int* positions, int T, int num_seqs, int H, int R,
                                         int D, int page_size, float scale, int window,
-                                        const float* sink, hipStream_t stream) {
+                                        const float* sink, int split_max_blocks,
+                                        hipStream_t stream) {
   RLIS_REQUIRE(T >= 0 && num_seqs > 0 && H > 0 && D >= R && max_pages > 0,
                "latent_attention_mfma: bad sizes");
   RLIS_REQUIRE(rlis_latent_attention_mfma_ok(R, D, page_size),
@@ -423,26 +475,36 @@ RLIS_API int rlis_latent_attention_mfma(const void* q, long long ldq, void* out,
   while (hp < H && hp < 16) hp *= 2;
   const int tb = 16 / hp;
   const int blocks = ceil_div(T, tb) + num_seqs;
-  dim3 grid(ceil_div(blocks, 4), ceil_div(H, hp));
-  RLIS_REQUIRE(grid.y <= 65535, "latent_attention_mfma: too many heads");
-  const int lds = 4 * 16 * (D + 8) * 2;
-#define LAUNCH(NT, slot)                                                                       \
+  const int heads_y = ceil_div(H, hp);
+  RLIS_REQUIRE(heads_y <= 65535, "latent_attention_mfma: too many heads");
+  // few blocks of columns (steps of few tokens): a workgroup's waves share one and split its keys
+  const bool split = (long long)blocks * heads_y <= split_max_blocks;
+  dim3 grid(split ? blocks : ceil_div(blocks, 4), heads_y);
+#define LAUNCH_AS(NT, SP, slot)                                                                \
   do {                                                                                         \
+    const int lds = SP ? 16 * (D + 8) * 2 + 2 * (4 * NT + 2) * kWave * 4                       \
+                       : 4 * 16 * (D + 8) * 2;                                                 \
     if (lds > 48 * 1024) {                                                                     \
       hipError_t e = grant_lds(g_latent_lds[slot],                                             \
-                               (const void*)latent_attention_mfma_kernel<NT>, lds);            \
+                               (const void*)latent_attention_mfma_kernel<NT, SP>, lds);        \
       RLIS_REQUIRE(e == hipSuccess, "latent_attention_mfma: LDS of %d bytes refused", lds);     \
     }                                                                                          \
-    latent_attention_mfma_kernel<NT><<<grid, 256, lds, stream>>>(                              \
+    latent_attention_mfma_kernel<NT, SP><<<grid, 256, lds, stream>>>(                          \
         (const bf16_t*)q, ldq, (bf16_t*)out, ldo, (const bf16_t*)pages, (const bf16_t*)pages_t, \
         block_tables, max_pages, cu, positions, num_seqs, H, R, D, page_size, scale, window,   \
         sink, hp);                                                                             \
+  } while (0)
+#define LAUNCH(NT, slot)                              \
+  do {                                                \
+    if (split) LAUNCH_AS(NT, true, 4 + slot);         \
+    else LAUNCH_AS(NT, false, slot);                  \
   } while (0)
   if (R <= 64) LAUNCH(4, 0);
   else if (R <= 128) LAUNCH(8, 1);
   else if (R <= 256) LAUNCH(16, 2);
   else LAUNCH(32, 3);
 #undef LAUNCH
+#undef LAUNCH_AS
   RLIS_LAUNCH_CHECK("latent_attention_mfma");
   return 0;
 }

@@ -84,7 +84,7 @@ def _cached_attention_case(dtype, H, d, r, R, n, page, seed):
     (3, 16, 8, 40, None, False), (2, 12, 6, 28, None, False), (4, 8, 0, 36, 16, True),
     (1, 24, 0, 70, 1, True), (2, 16, 0, 16, 33, False), (2, 32, 16, 128, 17, True),
     (20, 16, 16, 64, None, False), (16, 8, 0, 200, 40, True), (5, 16, 32, 288, None, True)])
-def test_attention_over_cached_latents(dtype, H, d, r, R, window, sink):
+def test_attention_over_cached_latents(dtype, H, d, r, R, window, sink, monkeypatch):
     """Cache write in two portions (pages in a shuffled order), then every query against the
     plain softmax over keys made from the latents: rotation, norm, window edges, the sink."""
     from rust_llm_inference_server_amd import ops
@@ -135,8 +135,11 @@ def test_attention_over_cached_latents(dtype, H, d, r, R, window, sink):
     if matrix:
         assert torch.equal(pages_t.transpose(1, 2), pages[:, :, :R])
         cu = torch.tensor([0, n], dtype=torch.int32, device=DEV)
-        got = ops.latent_attention(*args, pages_t=pages_t, cu=cu, num_seqs=1)
-        assert rel(got.reshape(n, H, R), want) < 3e-2
+        from rust_llm_inference_server_amd.ops import latent
+        for blocks in (1024, 0):         # a workgroup's waves share a block's keys, or do not
+            monkeypatch.setattr(latent, "LATENT_SPLIT_MAX_BLOCKS", blocks)
+            got = ops.latent_attention(*args, pages_t=pages_t, cu=cu, num_seqs=1)
+            assert rel(got.reshape(n, H, R), want) < 3e-2
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
