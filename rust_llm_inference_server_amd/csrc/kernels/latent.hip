@@ -277,7 +277,10 @@ RLIS_API int rlis_latent_attention(const void* q, int dtype, long long ldq, void
 // of the chunk, which puts a lane's 8 probabilities on 8 consecutive keys.  The queries wait in
 // LDS (a wave's own 16 rows); scale, mask, sink and sums are float32; P is rounded to
 // bfloat16 as the second product's operand only.  How a sequence's keys are cut follows from
-// its own positions, so a row does not depend on its neighbours.
+// its own positions, so a row does not depend on its neighbours.  A wave holds the sums of
+// 16 NT latent channels; wider latents are shared out over gridDim.z workgroups, each of which
+// forms the scores again (the walk is bound by the round trips of its loads, not by the matrix
+// cores, and fewer sums per wave leave registers for loads in flight).
 template <int NT, bool SPLIT>
 __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     const bf16_t* __restrict__ q, long long ldq, bf16_t* __restrict__ out, long long ldo,
@@ -323,6 +326,7 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
           *reinterpret_cast<const mma_u32x4*>(q_row + j);
   if (SPLIT) __syncthreads();
   const int* table = block_tables + (long long)seq * max_pages;
+  const int dim0 = blockIdx.z * NT * 16;         // this workgroup's share of the latent channels
   const bool opens = !SPLIT || wave == 0;        // whose sums the sink opens
   float m = (sink && opens) ? sink[head_c] : -INFINITY;
   float l = (sink && opens && g == 0) ? 1.f : 0.f;
@@ -331,7 +335,7 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
   for (int t = 0; t < NT; ++t) acc[t] = mma_f32x4{0.f, 0.f, 0.f, 0.f};
   const int steps = (D + 31) / 32;
   const mma_u32x4 zero = {0u, 0u, 0u, 0u};
-  constexpr int GS = NT >= 32 ? 4 : NT == 4 ? 4 : 6;     // key loads asked for together
+  constexpr int GS = NT == 4 ? 4 : 6;                    // key loads asked for together
   for (int k0 = (lo_blk & ~31) + (SPLIT ? 32 * wave : 0); k0 <= hi_blk;
        k0 += SPLIT ? 128 : 32) {
     const int kk0 = min(k0 + 8 * (c / 4) + c % 4, hi_blk), kk1 = min(kk0 + 4, hi_blk);
@@ -388,7 +392,7 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     const bf16_t* vt = pages_t + vpage * R * page_size + kv % page_size;
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-      const int dim = min(16 * t + c, R - 1);
+      const int dim = min(dim0 + 16 * t + c, R - 1);
       const mma_u32x4 a = *reinterpret_cast<const mma_u32x4*>(vt + (long long)dim * page_size);
       acc[t] *= corr;
       acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mma_bf16x8, a), pv,
@@ -439,7 +443,7 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
   for (int t = 0; t < NT; ++t)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int dim = 16 * t + 4 * g + i;
+      const int dim = dim0 + 16 * t + 4 * g + i;
       if (dim < R) o[dim] = f32_to_bf16(acc[t][i] * inv);
     }
 }
@@ -448,9 +452,7 @@ static LdsGrant g_latent_lds[8];
 
 // Whether the matrix-core kernel takes a latent of R numbers in rows of D.
 RLIS_API int rlis_latent_attention_mfma_ok(int R, int D, int page_size) {
-  if (R <= 0 || R > 512 || D % 8 || page_size % 8) return 0;
-  const int nt = R <= 64 ? 4 : R <= 128 ? 8 : R <= 256 ? 16 : 32;
-  return D <= 16 * nt + 64 ? 1 : 0;
+  return (R > 0 && R <= 4096 && D >= R && D <= 1536 && D % 8 == 0 && page_size % 8 == 0) ? 1 : 0;
 }
 
 RLIS_API int rlis_latent_attention_mfma(const void* q, long long ldq, void* out, long long ldo,
@@ -479,7 +481,10 @@ RLIS_API int rlis_latent_attention_mfma(const void* q, long long ldq, void* out,
   RLIS_REQUIRE(heads_y <= 65535, "latent_attention_mfma: too many heads");
   // few blocks of columns (steps of few tokens): a workgroup's waves share one and split its keys
   const bool split = (long long)blocks * heads_y <= split_max_blocks;
-  dim3 grid(split ? blocks : ceil_div(blocks, 4), heads_y);
+  // sums per wave: up to 128 latent channels
+  const int tiles = ceil_div(R, 16);
+  const int nt = tiles <= 4 ? 4 : 8;
+  dim3 grid(split ? blocks : ceil_div(blocks, 4), heads_y, ceil_div(tiles, nt));
 #define LAUNCH_AS(NT, SP, slot)                                                                \
   do {                                                                                         \
     const int lds = SP ? 16 * (D + 8) * 2 + 2 * (4 * NT + 2) * kWave * 4                       \
@@ -499,10 +504,8 @@ RLIS_API int rlis_latent_attention_mfma(const void* q, long long ldq, void* out,
     if (split) LAUNCH_AS(NT, true, 4 + slot);         \
     else LAUNCH_AS(NT, false, slot);                  \
   } while (0)
-  if (R <= 64) LAUNCH(4, 0);
-  else if (R <= 128) LAUNCH(8, 1);
-  else if (R <= 256) LAUNCH(16, 2);
-  else LAUNCH(32, 3);
+  if (nt == 4) LAUNCH(4, 0);
+  else LAUNCH(8, 1);
 #undef LAUNCH
 #undef LAUNCH_AS
   RLIS_LAUNCH_CHECK("latent_attention_mfma");

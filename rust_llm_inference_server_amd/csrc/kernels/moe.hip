@@ -220,6 +220,87 @@ __global__ __launch_bounds__(64 * WAVES) void moe_down_kernel(
   }
 }
 
+
+// The same two products for tiles of 64 rows (steps of many pairs): a wave takes all 64 rows of
+// the tile against columns of its own (gate/up: 32 of each, down: 64), so that every weight
+// fragment it loads serves four blocks of rows; the four waves of a workgroup take four
+// neighbouring column blocks of the same tile.  A row's sums are those of the small tiles.
+template <typename T, bool ALIGNED>
+__global__ __launch_bounds__(256) void moe_gate_up_rows_kernel(
+    const T* __restrict__ x, long long ldx, const T* __restrict__ w_gu,
+    const int* __restrict__ sorted, const int* __restrict__ tile_expert, int top, int F, int K,
+    T* __restrict__ hidden) {
+  const int e = tile_expert[blockIdx.x];
+  if (e < 0) return;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int row0 = blockIdx.x * 64;
+  const int f0 = (blockIdx.y * 4 + wave) * 32;
+  if (f0 >= F) return;
+  const T* a_row[4];
+#pragma unroll
+  for (int a = 0; a < 4; ++a) {
+    const int pair = sorted[row0 + a * 16 + lane % 16];
+    a_row[a] = x + (long long)(pair < 0 ? 0 : pair / top) * ldx;
+  }
+  const T* b_row[4];
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    const int f = min(f0 + (b & 1) * 16 + lane % 16, F - 1);
+    b_row[b] = w_gu + (((long long)e * 2 + (b >> 1)) * F + f) * K;
+  }
+  mma_f32x4 acc[4][4];
+  wave_tile_product_rows<T, 4, 4, ALIGNED>(a_row, b_row, K, acc);
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const int f = f0 + b * 16 + lane % 16;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int row = row0 + a * 16 + (lane / 16) * 4 + i;
+        const float g = acc[a][b][i], u = acc[a][b + 2][i];
+        if (f < F) st(hidden + (long long)row * F + f, g / (1.0f + expf(-g)) * u);
+      }
+    }
+}
+
+template <typename T, bool ALIGNED>
+__global__ __launch_bounds__(256) void moe_down_rows_kernel(
+    const T* __restrict__ hidden, const T* __restrict__ w_d, const int* __restrict__ sorted,
+    const int* __restrict__ tile_expert, const float* __restrict__ weights, int N, int F,
+    float* __restrict__ y) {
+  const int e = tile_expert[blockIdx.x];
+  if (e < 0) return;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int row0 = blockIdx.x * 64;
+  const int n0 = (blockIdx.y * 4 + wave) * 64;
+  if (n0 >= N) return;
+  const T* a_row[4];
+#pragma unroll
+  for (int a = 0; a < 4; ++a) a_row[a] = hidden + (long long)(row0 + a * 16 + lane % 16) * F;
+  const T* b_row[4];
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    const int n = min(n0 + b * 16 + lane % 16, N - 1);
+    b_row[b] = w_d + ((long long)e * N + n) * F;
+  }
+  mma_f32x4 acc[4][4];
+  wave_tile_product_rows<T, 4, 4, ALIGNED>(a_row, b_row, F, acc);
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int pair = sorted[row0 + a * 16 + (lane / 16) * 4 + i];
+      if (pair < 0) continue;
+      const float wt = weights[pair];
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const int n = n0 + b * 16 + lane % 16;
+        if (n < N) y[(long long)pair * N + n] = acc[a][b][i] * wt;
+      }
+    }
+}
+
 RLIS_API int rlis_moe_experts(const void* x, int dtype, long long ldx, const void* w_gu,
                               const void* w_d, const int* sorted, const int* tile_expert,
                               const float* weights, int tile_rows, int max_tiles, int top, int F,
@@ -232,10 +313,17 @@ RLIS_API int rlis_moe_experts(const void* x, int dtype, long long ldx, const voi
   dim3 g1(max_tiles, ceil_div(F, 32)), g2(max_tiles, ceil_div(K, 64));
 #define LAUNCH(T, WAVES, AL1, AL2)                                                             \
   do {                                                                                         \
-    moe_gate_up_kernel<T, WAVES, AL1><<<g1, 64 * WAVES, 0, stream>>>(                          \
-        (const T*)x, ldx, (const T*)w_gu, sorted, tile_expert, top, F, K, (T*)hidden);         \
-    moe_down_kernel<T, WAVES, AL2><<<g2, 64 * WAVES, 0, stream>>>(                             \
-        (const T*)hidden, (const T*)w_d, sorted, tile_expert, weights, K, F, y);               \
+    if (WAVES == 4) {                                                                          \
+      moe_gate_up_rows_kernel<T, AL1><<<dim3(max_tiles, ceil_div(F, 128)), 256, 0, stream>>>(  \
+          (const T*)x, ldx, (const T*)w_gu, sorted, tile_expert, top, F, K, (T*)hidden);       \
+      moe_down_rows_kernel<T, AL2><<<dim3(max_tiles, ceil_div(K, 256)), 256, 0, stream>>>(     \
+          (const T*)hidden, (const T*)w_d, sorted, tile_expert, weights, K, F, y);             \
+    } else {                                                                                   \
+      moe_gate_up_kernel<T, WAVES, AL1><<<g1, 64 * WAVES, 0, stream>>>(                        \
+          (const T*)x, ldx, (const T*)w_gu, sorted, tile_expert, top, F, K, (T*)hidden);       \
+      moe_down_kernel<T, WAVES, AL2><<<g2, 64 * WAVES, 0, stream>>>(                           \
+          (const T*)hidden, (const T*)w_d, sorted, tile_expert, weights, K, F, y);             \
+    }                                                                                          \
   } while (0)
 #define BY_ALIGN(T, WAVES)                                                                    \
   do {                                                                                        \

@@ -1031,28 +1031,50 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(
     a[j] = n < N ? -expf(a_log[(long long)c * N + n]) : 0.f;
   }
   const float bias = dt_bias[c], dsk = dskip[c];
-  for (int t = t0; t < t1; ++t) {
-    const float raw = dt_raw[(long long)t * lddt + c] + bias;
-    const float dt = raw > 20.f ? raw : log1pf(expf(raw));
-    const float xv = ld(x + (long long)t * ldx + c);
-    const float dx = dt * xv;
-    const float* bt = bmat + (long long)t * ldbc;
-    const float* ct = cmat + (long long)t * ldbc;
-    float y = 0.f;
+  // Tokens are walked in groups of kScanGroup: everything that does not depend on the state
+  // (a token's step, input, gate, B and C, and the decays exp(dt A)) is asked for and made for
+  // the whole group first, so that the walk itself waits for no load; tokens past the
+  // sequence's end take the last token's addresses and are not stored.
+  constexpr int G = NPL <= 8 ? 8 : 4;
+  for (int tg = t0; tg < t1; tg += G) {
+    float dtv[G], xv[G], zv[G], bn[G][NPL], cn[G][NPL];
 #pragma unroll
-    for (int j = 0; j < NPL; ++j) {
-      const int n = sub + j * LPC;
-      const int nn = n < N ? n : 0;
-      const float bn = bt[nn], cn = ct[nn];
-      const float v = expf(dt * a[j]) * st_[j] + dx * bn;
-      st_[j] = n < N ? v : 0.f;
-      y = fmaf(st_[j], cn, y);
+    for (int u = 0; u < G; ++u) {
+      const int t = min(tg + u, t1 - 1);
+      dtv[u] = dt_raw[(long long)t * lddt + c];
+      xv[u] = ld(x + (long long)t * ldx + c);
+      zv[u] = z[(long long)t * ldz + c];
+#pragma unroll
+      for (int j = 0; j < NPL; ++j) {
+        const int n = sub + j * LPC;
+        const int nn = n < N ? n : 0;
+        bn[u][j] = bmat[(long long)t * ldbc + nn];
+        cn[u][j] = cmat[(long long)t * ldbc + nn];
+      }
     }
 #pragma unroll
-    for (int o = 1; o < LPC; o <<= 1) y += __shfl_xor(y, o, kWave);
-    if (sub == 0) {
-      const float zv = z[(long long)t * ldz + c];
-      st(out + (long long)t * ldo + c, (y + dsk * xv) * (zv / (1.0f + expf(-zv))));
+    for (int u = 0; u < G; ++u) {
+      const float raw = dtv[u] + bias;
+      dtv[u] = raw > 20.f ? raw : log1pf(expf(raw));
+    }
+#pragma unroll
+    for (int u = 0; u < G; ++u) {
+      if (tg + u < t1) {                       // (the same for all lanes of a sequence)
+        const float dt = dtv[u], dx = dt * xv[u];
+        float y = 0.f;
+#pragma unroll
+        for (int j = 0; j < NPL; ++j) {
+          const int n = sub + j * LPC;
+          const float v = expf(dt * a[j]) * st_[j] + dx * bn[u][j];
+          st_[j] = n < N ? v : 0.f;
+          y = fmaf(st_[j], cn[u][j], y);
+        }
+#pragma unroll
+        for (int o = 1; o < LPC; o <<= 1) y += __shfl_xor(y, o, kWave);
+        if (sub == 0)
+          st(out + (long long)(tg + u) * ldo + c,
+             (y + dsk * xv[u]) * (zv[u] / (1.0f + expf(-zv[u]))));
+      }
     }
   }
 #pragma unroll

@@ -82,3 +82,42 @@ static inline bool mma_rows_aligned(const void* base, long long stride, long lon
   constexpr int n = MmaChunk<T>::kLane;
   return ((uintptr_t)base % 16 == 0) && stride % n == 0 && inner % n == 0 && K % n == 0;
 }
+
+// The same with MB blocks of 16 rows of A: acc[a][b] is block a of A against block b of B.  Every
+// fragment of B that is loaded serves MB products (and every fragment of A NB of them), which
+// is what a product with many rows needs: loads, not the matrix cores, bound the tile above.
+template <typename T, int MB, int NB, bool ALIGNED>
+__device__ __forceinline__ void wave_tile_product_rows(const T* const (&a_row)[MB],
+                                                       const T* const (&b_row)[NB], int K,
+                                                       mma_f32x4 (&acc)[MB][NB]) {
+  constexpr int kLane = MmaChunk<T>::kLane, kStep = MmaChunk<T>::kStep;
+  const int g = (threadIdx.x % kWave) / 16;
+#pragma unroll
+  for (int a = 0; a < MB; ++a)
+#pragma unroll
+    for (int b = 0; b < NB; ++b) acc[a][b] = mma_f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < K; k0 += kStep) {
+    const int k = k0 + g * kLane;
+    mma_u32x4 av[MB], bv[NB];
+#pragma unroll
+    for (int a = 0; a < MB; ++a) av[a] = mma_load<T, ALIGNED>(a_row[a], k, K);
+#pragma unroll
+    for (int b = 0; b < NB; ++b) bv[b] = mma_load<T, ALIGNED>(b_row[b], k, K);
+#pragma unroll
+    for (int a = 0; a < MB; ++a)
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        if constexpr (sizeof(T) == 2) {
+          acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              __builtin_bit_cast(mma_bf16x8, av[a]), __builtin_bit_cast(mma_bf16x8, bv[b]),
+              acc[a][b], 0, 0, 0);
+        } else {
+          const mma_f32x4 af = __builtin_bit_cast(mma_f32x4, av[a]);
+          const mma_f32x4 bf = __builtin_bit_cast(mma_f32x4, bv[b]);
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[i], bf[i], acc[a][b], 0, 0, 0);
+        }
+      }
+  }
+}

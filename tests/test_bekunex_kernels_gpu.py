@@ -83,7 +83,8 @@ def _cached_attention_case(dtype, H, d, r, R, n, page, seed):
 @pytest.mark.parametrize("H, d, r, R, window, sink", [
     (3, 16, 8, 40, None, False), (2, 12, 6, 28, None, False), (4, 8, 0, 36, 16, True),
     (1, 24, 0, 70, 1, True), (2, 16, 0, 16, 33, False), (2, 32, 16, 128, 17, True),
-    (20, 16, 16, 64, None, False), (16, 8, 0, 200, 40, True), (5, 16, 32, 288, None, True)])
+    (20, 16, 16, 64, None, False), (16, 8, 0, 200, 40, True), (5, 16, 32, 288, None, True),
+    (2, 8, 8, 520, 50, True)])
 def test_attention_over_cached_latents(dtype, H, d, r, R, window, sink, monkeypatch):
     """Cache write in two portions (pages in a shuffled order), then every query against the
     plain softmax over keys made from the latents: rotation, norm, window edges, the sink."""
