@@ -481,9 +481,10 @@ RLIS_API int rlis_latent_attention_mfma(const void* q, long long ldq, void* out,
   RLIS_REQUIRE(heads_y <= 65535, "latent_attention_mfma: too many heads");
   // few blocks of columns (steps of few tokens): a workgroup's waves share one and split its keys
   const bool split = (long long)blocks * heads_y <= split_max_blocks;
-  // sums per wave: up to 128 latent channels
+  // sums per wave: up to 128 latent channels in small steps (more workgroups, more loads in
+  // flight), up to 256 in large ones (the scores are formed once more per share)
   const int tiles = ceil_div(R, 16);
-  const int nt = tiles <= 4 ? 4 : 8;
+  const int nt = tiles <= 4 ? 4 : (tiles <= 8 || split) ? 8 : 16;
   dim3 grid(split ? blocks : ceil_div(blocks, 4), heads_y, ceil_div(tiles, nt));
 #define LAUNCH_AS(NT, SP, slot)                                                                \
   do {                                                                                         \
@@ -505,7 +506,8 @@ RLIS_API int rlis_latent_attention_mfma(const void* q, long long ldq, void* out,
     else LAUNCH_AS(NT, false, slot);                  \
   } while (0)
   if (nt == 4) LAUNCH(4, 0);
-  else LAUNCH(8, 1);
+  else if (nt == 8) LAUNCH(8, 1);
+  else LAUNCH(16, 2);
 #undef LAUNCH
 #undef LAUNCH_AS
   RLIS_LAUNCH_CHECK("latent_attention_mfma");

@@ -1036,6 +1036,27 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(
   // the whole group first, so that the walk itself waits for no load; tokens past the
   // sequence's end take the last token's addresses and are not stored.
   constexpr int G = NPL <= 8 ? 8 : 4;
+  if (t1 - t0 == 1) {                          // a decoded token: nothing to group
+    const int t = t0;
+    const float raw = dt_raw[(long long)t * lddt + c] + bias;
+    const float dt = raw > 20.f ? raw : log1pf(expf(raw));
+    const float xs = ld(x + (long long)t * ldx + c), dx = dt * xs;
+    float y = 0.f;
+#pragma unroll
+    for (int j = 0; j < NPL; ++j) {
+      const int n = sub + j * LPC;
+      const int nn = n < N ? n : 0;
+      const float v = expf(dt * a[j]) * st_[j] + dx * bmat[(long long)t * ldbc + nn];
+      st_[j] = n < N ? v : 0.f;
+      y = fmaf(st_[j], cmat[(long long)t * ldbc + nn], y);
+    }
+#pragma unroll
+    for (int o = 1; o < LPC; o <<= 1) y += __shfl_xor(y, o, kWave);
+    if (sub == 0) {
+      const float zs = z[(long long)t * ldz + c];
+      st(out + (long long)t * ldo + c, (y + dsk * xs) * (zs / (1.0f + expf(-zs))));
+    }
+  } else
   for (int tg = t0; tg < t1; tg += G) {
     float dtv[G], xv[G], zv[G], bn[G][NPL], cn[G][NPL];
 #pragma unroll
