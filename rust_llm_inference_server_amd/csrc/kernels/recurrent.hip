@@ -1009,6 +1009,20 @@ RLIS_API int rlis_head_norm_gate(void* out, int out_dtype, const float* o, const
 // are walked in order from the state its slot holds, which is left as after the last one.
 // x (the convolution's output) and the result are in the activation dtype; everything else,
 // the state included, is float32.
+// Sum over the LPC neighbouring lanes that share a channel (4, 16 or 64, aligned): adds between
+// lanes of a row of 16 by data-parallel primitives, no trip through LDS; every lane gets it.
+template <int LPC>
+__device__ __forceinline__ float channel_sum(float v) {
+  if (LPC == 64) return lanes_sum(v);
+  v += dpp_from<0xB1>(v);      // quad_perm [1, 0, 3, 2]
+  v += dpp_from<0x4E>(v);      // quad_perm [2, 3, 0, 1]
+  if (LPC == 16) {
+    v += dpp_from<0x141>(v);   // row_half_mirror
+    v += dpp_from<0x140>(v);   // row_mirror
+  }
+  return v;
+}
+
 template <typename TO, int NPL, int LPC>
 __global__ __launch_bounds__(256) void selective_scan_kernel(
     TO* __restrict__ out, long long ldo, const TO* __restrict__ x, long long ldx,
@@ -1050,8 +1064,7 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(
       st_[j] = n < N ? v : 0.f;
       y = fmaf(st_[j], cmat[(long long)t * ldbc + nn], y);
     }
-#pragma unroll
-    for (int o = 1; o < LPC; o <<= 1) y += __shfl_xor(y, o, kWave);
+    y = channel_sum<LPC>(y);
     if (sub == 0) {
       const float zs = z[(long long)t * ldz + c];
       st(out + (long long)t * ldo + c, (y + dsk * xs) * (zs / (1.0f + expf(-zs))));
@@ -1090,8 +1103,7 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(
           st_[j] = n < N ? v : 0.f;
           y = fmaf(st_[j], cn[u][j], y);
         }
-#pragma unroll
-        for (int o = 1; o < LPC; o <<= 1) y += __shfl_xor(y, o, kWave);
+        y = channel_sum<LPC>(y);
         if (sub == 0)
           st(out + (long long)(tg + u) * ldo + c,
              (y + dsk * xv[u]) * (zv[u] / (1.0f + expf(-zv[u]))));
@@ -1111,7 +1123,7 @@ RLIS_API int rlis_selective_scan(void* out, int out_dtype, long long ldo, const 
                                  long long ldbc, const float* z, long long ldz,
                                  const float* a_log, const float* dskip, float* state,
                                  long long state_stride, const int* cu, const int* slots,
-                                 int num_seqs, int C, int N, hipStream_t stream) {
+                                 int num_seqs, int C, int N, int long_runs, hipStream_t stream) {
   RLIS_REQUIRE(num_seqs >= 0 && C > 0 && N > 0, "selective_scan: bad sizes C=%d N=%d", C, N);
   RLIS_REQUIRE(N <= 1024, "selective_scan: a state of %d numbers per channel is too large", N);
   RLIS_REQUIRE(ldo >= C && ldx >= C && lddt >= C && ldz >= C && ldbc >= N &&
@@ -1123,9 +1135,14 @@ RLIS_API int rlis_selective_scan(void* out, int out_dtype, long long ldo, const 
   selective_scan_kernel<TO, NPL, LPC><<<dim3(ceil_div(C * LPC, 256), num_seqs), 256, 0, stream>>>( \
       (TO*)out, ldo, (const TO*)x, ldx, dt_raw, lddt, dt_bias, bmat, cmat, ldbc, z, ldz, a_log, dskip,   \
       state, state_stride, cu, slots, C, N)
+  // long_runs: sequences bring many tokens each and there are few of them, so a channel's states
+  // are spread over more lanes (more waves on a chip that the walk leaves mostly idle); the sum
+  // over the states is then added up in another order
 #define BY_N(TO)                                  \
   do {                                            \
-    if (N <= 16) LAUNCH(TO, 4, 4);                \
+    if (N <= 16 && long_runs) LAUNCH(TO, 1, 16);  \
+    else if (N <= 16) LAUNCH(TO, 4, 4);           \
+    else if (N <= 64 && long_runs) LAUNCH(TO, 4, 16); \
     else if (N <= 32) LAUNCH(TO, 8, 4);           \
     else if (N <= 64) LAUNCH(TO, 16, 4);          \
     else if (N <= 256) LAUNCH(TO, 16, 16);        \

@@ -220,6 +220,13 @@ def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, he
     return out
 
 
+# A step whose sequences bring at least this many tokens on average, and together at most this
+# many channels, spreads a channel's states over sixteen lanes instead of four (known from the
+# host: the number of rows and of sequences).
+SPREAD_SCAN_MIN_MEAN_TOKENS = 64
+SPREAD_SCAN_MAX_CHANNELS = 65536
+
+
 def selective_scan(x: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, b: torch.Tensor,
                    c: torch.Tensor, z: torch.Tensor, a_log: torch.Tensor, skip: torch.Tensor,
                    state: torch.Tensor, cu: torch.Tensor, slots: torch.Tensor,
@@ -252,5 +259,6 @@ def selective_scan(x: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor,
                                                          "selective_scan A_log"),
              _vec(skip, C, "selective_scan skip"), state.data_ptr(), stride,
              _meta(cu, num_seqs + 1, "cu"), _meta(slots, num_seqs, "slots"), num_seqs, C, N,
-             lib.stream_ptr())
+             int(T >= SPREAD_SCAN_MIN_MEAN_TOKENS * max(1, num_seqs)
+                 and num_seqs * C <= SPREAD_SCAN_MAX_CHANNELS), lib.stream_ptr())
     return out

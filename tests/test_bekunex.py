@@ -401,3 +401,31 @@ def test_the_replay_program_runs_the_model(dtype_name, tmp_path_factory, tmp_pat
         want = plain.forward(stored, cfg, tokens)
         errors += [bm.row_error(row, want[pos]) for pos, row in got[rid].items()]
     bm.judge(errors, dtype_name)
+
+
+@pytest.mark.gpu
+def test_the_command_line_generates_and_scores(tmp_path_factory, tmp_path, capsys):
+    """``rlis generate`` picks the design by config.json and prints the plain implementation's
+    greedy tokens; ``rlis perplexity`` scores a token file through the same step function."""
+    from rust_llm_inference_server_amd import cli
+    folder, cfg, stored = model_case("b", "float32", tmp_path_factory)
+    prompt = bm.prompts(cfg["vocab"], [11], seed=20)[0]
+    rc = cli.main(["generate", "--model", folder, "--dtype", "f32", "--max-seq-len", "128",
+                   "--num-pages", "32", "--block-size", "8", "--max-num-seqs", "2",
+                   "--max-tokens", "5", "--prompt-ids", ",".join(map(str, prompt))])
+    out = capsys.readouterr()
+    assert rc == 0
+    got = [int(t) for t in out.out.split()]
+    tokens = list(prompt)
+    for g in got:
+        last = plain.forward(stored, cfg, tokens)[-1]
+        best = int(torch.argmax(last))
+        assert g == best or float(last[best] - last[g]) < 1e-3
+        tokens.append(g)
+    assert len(got) == 5 and "output 5 tok (length)" in out.err
+    ids = tmp_path / "ids.txt"
+    ids.write_text(" ".join(map(str, bm.prompts(cfg["vocab"], [96], seed=21)[0])))
+    rc = cli.main(["perplexity", "--model", folder, "--dtype", "f32", "--max-seq-len", "128",
+                   "--ids-file", str(ids), "--ctx", "32"])
+    out = capsys.readouterr()
+    assert rc == 0 and json.loads(out.out.strip().splitlines()[-1])["ppl"] > 1.0
