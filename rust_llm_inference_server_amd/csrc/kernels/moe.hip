@@ -12,6 +12,7 @@
 //  * moe_gate_up / moe_down: the units' products on the matrix cores, tile by tile
 //    (tile_mma.h), rows gathered through the sorted list; silu(gate) * up in the epilogue of the
 //    first, the pair's weight in the epilogue of the second.
+//    Steps of thousands of pairs take tiles of 128 rows staged through LDS (moe_tiles128).
 //  * moe_combine: a token's pairs added in the order of its choices, plus an optional addend
 //    (a shared unit that every token takes), float32.
 #include "common.h"
@@ -301,14 +302,154 @@ __global__ __launch_bounds__(256) void moe_down_rows_kernel(
     }
 }
 
+// ------------------------------------------------- tiles of 128 rows through LDS (bfloat16)
+// For steps of thousands of pairs: the dense matrix-core product's cut (tile 128 x 128 x 64,
+// both operands staged through LDS with the next k slab in registers meanwhile, four waves of
+// 64 x 64 as 2 x 2 blocks of v_mfma_f32_32x32x16_bf16) with a tile's rows gathered through the
+// sorted list and its weights taken from the tile's expert.  GATE_UP: the 128 weight rows of a
+// tile are [gate f..f+31 | up f..f+31 | gate f+32..f+63 | up f+32..f+63], so that a wave holds
+// gate and up of the same 32 columns and stores silu(gate) * up; otherwise the result times
+// the pair's weight goes to the pair's row of y.
+typedef float moe_f32x16 __attribute__((ext_vector_type(16)));
+
+template <bool GATE_UP>
+__global__ __launch_bounds__(256) void moe_tiles128_kernel(
+    const bf16_t* __restrict__ A, long long lda, const bf16_t* __restrict__ W,
+    const int* __restrict__ sorted, const int* __restrict__ tile_expert,
+    const float* __restrict__ weights, int top, int N, int K, bf16_t* __restrict__ hidden,
+    float* __restrict__ y) {
+  constexpr int BM = 128, BK = 64, LDS_STRIDE = BK + 8;
+  __shared__ __attribute__((aligned(16))) bf16_t As[BM * LDS_STRIDE];
+  __shared__ __attribute__((aligned(16))) bf16_t Bs[BM * LDS_STRIDE];
+  const int e = tile_expert[blockIdx.x];
+  if (e < 0) return;
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  const int wm = wave / 2, wn = wave % 2;
+  const int row0 = blockIdx.x * BM;
+  const int n0 = blockIdx.y * (GATE_UP ? 64 : 128);
+  // the rows this thread moves: chunk c = tid + 256 i covers tile row c / 8, k offset (c % 8) * 8
+  const bf16_t* a_src[4];
+  const bf16_t* b_src[4];
+  bool b_ok[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = (tid + i * 256) / 8;
+    if (GATE_UP) {
+      const int pair = sorted[row0 + r];
+      a_src[i] = A + (long long)(pair < 0 ? 0 : pair / top) * lda;
+      const int f = n0 + (r / 64) * 32 + r % 32;
+      b_ok[i] = f < N;
+      b_src[i] = W + (((long long)e * 2 + (r / 32) % 2) * N + (b_ok[i] ? f : 0)) * K;
+    } else {
+      a_src[i] = A + (long long)(row0 + r) * lda;
+      const int n = n0 + r;
+      b_ok[i] = n < N;
+      b_src[i] = W + ((long long)e * N + (b_ok[i] ? n : 0)) * K;
+    }
+  }
+  moe_f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  mma_u32x4 ra[4], rb[4];
+  const mma_u32x4 zero = {0u, 0u, 0u, 0u};
+  auto load_global = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int gk = k0 + ((tid + i * 256) % 8) * 8;
+      const mma_u32x4 va = *reinterpret_cast<const mma_u32x4*>(a_src[i] + (gk < K ? gk : 0));
+      const mma_u32x4 vb = *reinterpret_cast<const mma_u32x4*>(b_src[i] + (gk < K ? gk : 0));
+      ra[i] = gk < K ? va : zero;
+      rb[i] = (gk < K && b_ok[i]) ? vb : zero;
+    }
+  };
+  auto store_lds = [&]() {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = tid + i * 256;
+      *reinterpret_cast<mma_u32x4*>(As + (c / 8) * LDS_STRIDE + (c % 8) * 8) = ra[i];
+      *reinterpret_cast<mma_u32x4*>(Bs + (c / 8) * LDS_STRIDE + (c % 8) * 8) = rb[i];
+    }
+  };
+  const int num_k = (K + BK - 1) / BK;
+  load_global(0);
+  store_lds();
+  __syncthreads();
+  for (int kt = 0; kt < num_k; ++kt) {
+    if (kt + 1 < num_k) load_global((kt + 1) * BK);
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      mma_bf16x8 a[2], b[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        a[i] = *reinterpret_cast<const mma_bf16x8*>(
+            As + (wm * 64 + i * 32 + lane % 32) * LDS_STRIDE + ks * 16 + (lane / 32) * 8);
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        b[j] = *reinterpret_cast<const mma_bf16x8*>(
+            Bs + (wn * 64 + j * 32 + lane % 32) * LDS_STRIDE + ks * 16 + (lane / 32) * 8);
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    __syncthreads();
+    if (kt + 1 < num_k) {
+      store_lds();
+      __syncthreads();
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = row0 + wm * 64 + i * 32 + (r / 4) * 8 + (lane / 32) * 4 + r % 4;
+      if (GATE_UP) {
+        const int f = n0 + wn * 32 + lane % 32;
+        const float g = acc[i][0][r], u = acc[i][1][r];
+        if (f < N) hidden[(long long)row * N + f] = f32_to_bf16(g / (1.0f + expf(-g)) * u);
+      } else {
+        const int pair = sorted[row];
+        if (pair < 0) continue;
+        const float wt = weights[pair];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int n = n0 + wn * 64 + j * 32 + lane % 32;
+          if (n < N) y[(long long)pair * N + n] = acc[i][j][r] * wt;
+        }
+      }
+    }
+}
+
 RLIS_API int rlis_moe_experts(const void* x, int dtype, long long ldx, const void* w_gu,
                               const void* w_d, const int* sorted, const int* tile_expert,
                               const float* weights, int tile_rows, int max_tiles, int top, int F,
                               int K, void* hidden, float* y, hipStream_t stream) {
-  RLIS_REQUIRE((tile_rows == 16 || tile_rows == 64) && max_tiles >= 0 && top > 0 && F > 0 && K > 0,
+  RLIS_REQUIRE((tile_rows == 16 || tile_rows == 64 || tile_rows == 128) && max_tiles >= 0 &&
+                   top > 0 && F > 0 && K > 0,
                "moe_experts: bad sizes");
   RLIS_REQUIRE(ldx >= K, "moe_experts: row stride shorter than a row");
   if (max_tiles == 0) return 0;
+  if (tile_rows == 128) {
+    RLIS_REQUIRE(dtype == RLIS_BF16 && mma_rows_aligned<bf16_t>(x, ldx, 0, K) &&
+                     mma_rows_aligned<bf16_t>(w_gu, K, 0, K) &&
+                     mma_rows_aligned<bf16_t>(hidden, F, 0, F) &&
+                     mma_rows_aligned<bf16_t>(w_d, F, 0, F),
+                 "moe_experts: tiles of 128 rows take bfloat16 rows on 16-byte boundaries");
+    RLIS_REQUIRE(ceil_div(F, 64) <= 65535 && ceil_div(K, 128) <= 65535, "moe_experts: too wide");
+    moe_tiles128_kernel<true><<<dim3(max_tiles, ceil_div(F, 64)), 256, 0, stream>>>(
+        (const bf16_t*)x, ldx, (const bf16_t*)w_gu, sorted, tile_expert, weights, top, F, K,
+        (bf16_t*)hidden, nullptr);
+    moe_tiles128_kernel<false><<<dim3(max_tiles, ceil_div(K, 128)), 256, 0, stream>>>(
+        (const bf16_t*)hidden, F, (const bf16_t*)w_d, sorted, tile_expert, weights, top, K, F,
+        nullptr, y);
+    RLIS_LAUNCH_CHECK("moe_experts");
+    return 0;
+  }
   RLIS_REQUIRE(ceil_div(F, 32) <= 65535 && ceil_div(K, 64) <= 65535, "moe_experts: too wide");
   dim3 g1(max_tiles, ceil_div(F, 32)), g2(max_tiles, ceil_div(K, 64));
 #define LAUNCH(T, WAVES, AL1, AL2)                                                             \

@@ -17,6 +17,9 @@ _DT = {torch.float32: 0, torch.bfloat16: 1}
 # Steps with at most this many (token, expert) pairs take tiles of 16 rows, larger ones of 64: a
 # row's sums are the same either way.
 SMALL_TILE_MAX_PAIRS = 256
+# bfloat16 steps with at least this many pairs per expert on average take tiles of 128 rows that
+# are staged through LDS (another matrix instruction: a row's sums agree to rounding).
+LARGE_TILE_MIN_PAIRS_PER_EXPERT = 96
 
 
 def route(logits: torch.Tensor, correction: torch.Tensor, groups: int, keep: int, top: int,
@@ -68,6 +71,9 @@ def routed_units(x: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor,
         return out
     P = T * top
     rows = 16 if P <= SMALL_TILE_MAX_PAIRS else 64
+    if x.dtype == torch.bfloat16 and P >= LARGE_TILE_MIN_PAIRS_PER_EXPERT * E and W % 8 == 0 \
+            and F % 8 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0:
+        rows = 128
     tiles = min(P, -(-(P + E * (rows - 1)) // rows))
     order = torch.empty(tiles * rows, dtype=torch.int32, device=x.device)
     tile_expert = torch.empty(tiles, dtype=torch.int32, device=x.device)

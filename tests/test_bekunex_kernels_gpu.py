@@ -172,10 +172,12 @@ def test_the_choice_of_experts(E, G, keep, top):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("T, E, top, W, F", [(1, 4, 2, 48, 24), (9, 8, 3, 40, 20),
-                                             (200, 6, 2, 64, 32), (77, 3, 1, 36, 12)])
+                                             (200, 6, 2, 64, 32), (77, 3, 1, 36, 12),
+                                             (700, 4, 2, 72, 40), (1000, 3, 3, 200, 136)])
 def test_routed_units(dtype, T, E, top, W, F):
-    """Tiles of 16 rows (few pairs) and of 64 (many), widths on and off the 16-byte loads, with
-    and without an addend; experts that no token chose."""
+    """Tiles of 16 rows (few pairs), of 64 (many) and, in bfloat16, of 128 through LDS (very
+    many), widths on and off the 16-byte loads and the tiles' sizes, with and without an addend;
+    experts that no token chose."""
     from rust_llm_inference_server_amd import ops
     x = rnd(T, W, seed=T).to(dtype)
     wgu = rnd(E, 2 * F, W, seed=T + 1, std=W ** -0.5).to(dtype)
