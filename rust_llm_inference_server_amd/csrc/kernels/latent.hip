@@ -448,7 +448,175 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     }
 }
 
+// The same walk for steps of many tokens, with a chunk's keys and values staged once per
+// workgroup: 4 DH waves, wave (cb, dh) taking column block cb (of four neighbouring ones: 4 x 16
+// / HP tokens of one sequence) and the share dh of the latent channels (16 NT each).  All
+// threads ask for the next chunk's rows together (one round trip, in flight during the
+// products of the chunk at hand), park them in registers and move them to LDS behind a barrier;
+// every fragment of a key or a value that was loaded once then serves the four column blocks.
+// The arithmetic of a column is that of the kernel above (the two shares of a column block form
+// the same scores and statistics).
+template <int NT, int DH>
+__global__ __launch_bounds__(256 * DH) void latent_attention_staged_kernel(
+    const bf16_t* __restrict__ q, long long ldq, bf16_t* __restrict__ out, long long ldo,
+    const bf16_t* __restrict__ pages, const bf16_t* __restrict__ pages_t,
+    const int* __restrict__ block_tables, int max_pages, const int* __restrict__ cu,
+    const int* __restrict__ positions, int num_seqs, int H, int R, int D, int page_size,
+    float scale, int window, const float* __restrict__ sink, int HP) {
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  constexpr int THREADS = 256 * DH, VD = NT * 16 * DH, VSTRIDE = 40;
+  constexpr int KL = DH == 2 ? 5 : 6, VL = NT / 4;
+  const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+  const int c = lane % 16, g = lane / 16;
+  const int cb = wave % 4, dh = wave / 4;
+  const int TB = 16 / HP;
+  const int stride = D + 8;
+  bf16_t* q_s = reinterpret_cast<bf16_t*>(lds_raw) + (size_t)cb * 16 * stride;
+  bf16_t* k_s = reinterpret_cast<bf16_t*>(lds_raw) + (size_t)64 * stride;
+  bf16_t* v_s = k_s + (size_t)32 * stride;
+  int blk = blockIdx.x;
+  int seq = -1, t_first = 0, t_end = 0;
+  for (int s = 0; s < num_seqs; ++s) {
+    const int a = cu[s], b = cu[s + 1];
+    const int tiles = (b - a + 4 * TB - 1) / (4 * TB);
+    if (blk < tiles) {
+      seq = s;
+      t_first = a + blk * 4 * TB;
+      t_end = b;
+      break;
+    }
+    blk -= tiles;
+  }
+  if (seq < 0) return;                               // (the whole workgroup)
+  const int tok = t_first + cb * TB + c / HP;
+  const int head = blockIdx.y * HP + c % HP;
+  const bool col_ok = tok < t_end && head < H;
+  const int tok_c = min(tok, t_end - 1), head_c = min(head, H - 1);
+  const int pos = positions[tok_c];
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int hi_wg = positions[min(t_first + 4 * TB, t_end) - 1];
+  const int p_first = positions[t_first];
+  const int lo_wg = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
+  if (dh == 0) {
+    const bf16_t* q_row = q + (long long)tok_c * ldq + (long long)head_c * D;
+    for (int j = g * 8; j < D; j += 32)
+      *reinterpret_cast<mma_u32x4*>(q_s + c * stride + j) =
+          *reinterpret_cast<const mma_u32x4*>(q_row + j);
+  }
+  const int* table = block_tables + (long long)seq * max_pages;
+  const int dim0 = blockIdx.z * VD + dh * NT * 16;   // this wave's latent channels
+  float m = sink ? sink[head_c] : -INFINITY;
+  float l = (sink && g == 0) ? 1.f : 0.f;
+  mma_f32x4 acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) acc[t] = mma_f32x4{0.f, 0.f, 0.f, 0.f};
+  const int steps = (D + 31) / 32;
+  const int segs = D / 8, k_total = 32 * segs;
+  const mma_u32x4 zero = {0u, 0u, 0u, 0u};
+  mma_u32x4 pk[KL], pv[VL];
+  // every thread's share of a chunk: KL 16-byte pieces of key rows, VL of value rows
+  auto ask = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < KL; ++i) {
+      const int idx = min(tid + i * THREADS, k_total - 1);
+      const int key = min(k0 + idx / segs, hi_wg);
+      pk[i] = *reinterpret_cast<const mma_u32x4*>(
+          pages + ((long long)table[key / page_size] * page_size + key % page_size) * D +
+          (idx % segs) * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < VL; ++i) {
+      const int idx = tid + i * THREADS;             // < VD * 4
+      const int key0 = k0 + 8 * (idx % 4);
+      const long long page = table[min(key0 / page_size, max_pages - 1)];
+      const int dim = min(blockIdx.z * VD + idx / 4, R - 1);
+      pv[i] = *reinterpret_cast<const mma_u32x4*>(pages_t + (page * R + dim) * page_size +
+                                                  key0 % page_size);
+    }
+  };
+  auto park = [&]() {
+#pragma unroll
+    for (int i = 0; i < KL; ++i) {
+      const int idx = tid + i * THREADS;
+      if (idx < k_total)
+        *reinterpret_cast<mma_u32x4*>(k_s + (idx / segs) * stride + (idx % segs) * 8) = pk[i];
+    }
+#pragma unroll
+    for (int i = 0; i < VL; ++i) {
+      const int idx = tid + i * THREADS;
+      *reinterpret_cast<mma_u32x4*>(v_s + (idx / 4) * VSTRIDE + (idx % 4) * 8) = pv[i];
+    }
+  };
+  const int k_first = lo_wg & ~31;
+  ask(k_first);
+  for (int k0 = k_first; k0 <= hi_wg; k0 += 32) {
+    __syncthreads();                                 // the chunk before has been read
+    park();
+    __syncthreads();
+    if (k0 + 32 <= hi_wg) ask(k0 + 32);
+    const bf16_t* kr0 = k_s + (8 * (c / 4) + c % 4) * stride;
+    const bf16_t* kr1 = kr0 + 4 * stride;
+    mma_f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < steps; ++s) {
+      const int dch = 32 * s + 8 * g;
+      const int at = dch < D ? dch : 0;
+      const mma_u32x4 qr = *reinterpret_cast<const mma_u32x4*>(q_s + c * stride + at);
+      const mma_u32x4 r0 = *reinterpret_cast<const mma_u32x4*>(kr0 + at);
+      const mma_u32x4 r1 = *reinterpret_cast<const mma_u32x4*>(kr1 + at);
+      const mma_bf16x8 qv = __builtin_bit_cast(mma_bf16x8, dch < D ? qr : zero);
+      s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+          __builtin_bit_cast(mma_bf16x8, dch < D ? r0 : zero), qv, s0, 0, 0, 0);
+      s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+          __builtin_bit_cast(mma_bf16x8, dch < D ? r1 : zero), qv, s1, 0, 0, 0);
+    }
+    float sv[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int key0 = k0 + 8 * g + i, key1 = key0 + 4;
+      sv[i] = (col_ok && key0 >= lo && key0 <= pos) ? s0[i] * scale : -INFINITY;
+      sv[4 + i] = (col_ok && key1 >= lo && key1 <= pos) ? s1[i] * scale : -INFINITY;
+      mx = fmaxf(mx, fmaxf(sv[i], sv[4 + i]));
+    }
+    mx = xor32_max(xor16_max(mx));
+    const float m_new = fmaxf(m, mx);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float corr = m == -INFINITY ? 0.f : __expf(m - m_use);
+    float psum = 0.f;
+    bf16_t pb[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float p = __expf(sv[j] - m_use);
+      psum += p;
+      pb[j] = f32_to_bf16(p);
+    }
+    l = l * corr + psum;
+    m = m_new;
+    const mma_bf16x8 pr = __builtin_bit_cast(mma_bf16x8, pb);
+    const bf16_t* vt = v_s + (size_t)(dh * NT * 16 + c) * VSTRIDE + 8 * g;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const mma_u32x4 a = *reinterpret_cast<const mma_u32x4*>(vt + (size_t)16 * t * VSTRIDE);
+      acc[t] *= corr;
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mma_bf16x8, a), pr,
+                                                       acc[t], 0, 0, 0);
+    }
+  }
+  const float total = xor32_sum(xor16_sum(l));
+  if (!col_ok) return;
+  const float inv = 1.0f / total;
+  bf16_t* o = out + (long long)tok * ldo + (long long)head * R;
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int dim = dim0 + 16 * t + 4 * g + i;
+      if (dim < R) o[dim] = f32_to_bf16(acc[t][i] * inv);
+    }
+}
+
 static LdsGrant g_latent_lds[8];
+static LdsGrant g_latent_staged_lds[3];
 
 // Whether the matrix-core kernel takes a latent of R numbers in rows of D.
 RLIS_API int rlis_latent_attention_mfma_ok(int R, int D, int page_size) {
@@ -460,7 +628,7 @@ RLIS_API int rlis_latent_attention_mfma(const void* q, long long ldq, void* out,
                                         const int* block_tables, int max_pages, const int* cu,
                                         const int* positions, int T, int num_seqs, int H, int R,
                                         int D, int page_size, float scale, int window,
-                                        const float* sink, int split_max_blocks,
+                                        const float* sink, int split_max_blocks, int staged,
                                         hipStream_t stream) {
   RLIS_REQUIRE(T >= 0 && num_seqs > 0 && H > 0 && D >= R && max_pages > 0,
                "latent_attention_mfma: bad sizes");
@@ -481,6 +649,36 @@ RLIS_API int rlis_latent_attention_mfma(const void* q, long long ldq, void* out,
   RLIS_REQUIRE(heads_y <= 65535, "latent_attention_mfma: too many heads");
   // few blocks of columns (steps of few tokens): a workgroup's waves share one and split its keys
   const bool split = (long long)blocks * heads_y <= split_max_blocks;
+  if (!split && staged && D <= 640) {
+    // large steps: a chunk's keys and values staged once per workgroup of four column blocks
+    const int tiles16 = ceil_div(R, 16);
+    const int wgs = ceil_div(T, 4 * tb) + num_seqs;
+#define STAGED(NT, DH, slot)                                                                     \
+  do {                                                                                           \
+    const int vd = NT * 16 * DH;                                                                 \
+    const int lds = (64 + 32) * (D + 8) * 2 + vd * 40 * 2;                                       \
+    if (lds > 48 * 1024) {                                                                       \
+      hipError_t e = grant_lds(g_latent_staged_lds[slot],                                        \
+                               (const void*)latent_attention_staged_kernel<NT, DH>, lds);        \
+      RLIS_REQUIRE(e == hipSuccess, "latent_attention_mfma: LDS of %d bytes refused", lds);       \
+    }                                                                                            \
+    latent_attention_staged_kernel<NT, DH>                                                       \
+        <<<dim3(wgs, heads_y, ceil_div(R, vd)), 256 * DH, lds, stream>>>(                        \
+            (const bf16_t*)q, ldq, (bf16_t*)out, ldo, (const bf16_t*)pages,                      \
+            (const bf16_t*)pages_t, block_tables, max_pages, cu, positions, num_seqs, H, R, D,   \
+            page_size, scale, window, sink, hp);                                                 \
+  } while (0)
+    bool took = true;
+    if (tiles16 > 16) STAGED(16, 2, 0);
+    else if (tiles16 > 8 && D <= 384) STAGED(16, 1, 1);
+    else if (tiles16 <= 8 && D <= 384) STAGED(8, 1, 2);
+    else took = false;
+#undef STAGED
+    if (took) {
+      RLIS_LAUNCH_CHECK("latent_attention_mfma");
+      return 0;
+    }
+  }
   // sums per wave: up to 128 latent channels in small steps (more workgroups, more loads in
   // flight), up to 256 in large ones (the scores are formed once more per share)
   const int tiles = ceil_div(R, 16);

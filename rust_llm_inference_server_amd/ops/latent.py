@@ -125,6 +125,9 @@ LATENT_ATTENTION = "matrix"
 # heads alone) let the four waves of a workgroup share a block and split its keys; larger steps
 # give every wave a block of its own.  The two differ in the order of the last additions.
 LATENT_SPLIT_MAX_BLOCKS = 1024
+# Larger steps stage a chunk's keys and values once per workgroup of four column blocks
+# (False: every wave loads its own).
+LATENT_STAGED = True
 
 
 def latent_mfma_ok(dtype: torch.dtype, rank: int, row: int, page_size: int = 16) -> bool:
@@ -174,7 +177,7 @@ def latent_attention(q: torch.Tensor, pages: torch.Tensor, block_tables: torch.T
                  block_tables.shape[1], _i32(cu, num_seqs + 1, "cu"),
                  _i32(positions, T, "positions"), T, int(num_seqs), heads, rank, D, page_size,
                  float(scale), int(window or 0), None if sink is None else sink.data_ptr(),
-                 int(LATENT_SPLIT_MAX_BLOCKS), lib.stream_ptr())
+                 int(LATENT_SPLIT_MAX_BLOCKS), int(LATENT_STAGED), lib.stream_ptr())
         return out
     lib.call("rlis_latent_attention", q.data_ptr(), _DT[q.dtype], ldq, out.data_ptr(),
              heads * rank, pages.data_ptr(), block_tables.data_ptr(), block_tables.shape[1],

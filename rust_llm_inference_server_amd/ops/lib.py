@@ -32,7 +32,7 @@ _SIGNATURES = {
     "rlis_scale": [P, I, L, F, P],
     "rlis_head_linear": [P, I, L, I, P, P, I, L, I, I, I, I, I, P],
     "rlis_latent_write": [P, L, P, F, I, I, I, P, P, P, P, P, P, I, I, I, P, L, I, I, P, L, I, I, I, P],
-    "rlis_latent_attention_mfma": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, I, F, I, P, I, P],
+    "rlis_latent_attention_mfma": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, I, F, I, P, I, I, P],
     "rlis_latent_attention": [P, I, L, P, L, P, P, I, P, P, I, I, I, I, I, F, I, P, P],
     "rlis_sigmoid_gate": [P, L, P, L, I, I, I, P],
     "rlis_moe_route": [P, L, P, I, I, I, I, I, F, P, P, P],

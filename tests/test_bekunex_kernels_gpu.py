@@ -137,8 +137,11 @@ def test_attention_over_cached_latents(dtype, H, d, r, R, window, sink, monkeypa
         assert torch.equal(pages_t.transpose(1, 2), pages[:, :, :R])
         cu = torch.tensor([0, n], dtype=torch.int32, device=DEV)
         from rust_llm_inference_server_amd.ops import latent
-        for blocks in (1024, 0):         # a workgroup's waves share a block's keys, or do not
+        # a workgroup's waves share a block's keys; every wave loads for itself; a workgroup
+        # stages a chunk once for four blocks
+        for blocks, staged in ((1024, False), (0, False), (0, True)):
             monkeypatch.setattr(latent, "LATENT_SPLIT_MAX_BLOCKS", blocks)
+            monkeypatch.setattr(latent, "LATENT_STAGED", staged)
             got = ops.latent_attention(*args, pages_t=pages_t, cu=cu, num_seqs=1)
             assert rel(got.reshape(n, H, R), want) < 3e-2
 
