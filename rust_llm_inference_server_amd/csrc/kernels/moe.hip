@@ -20,6 +20,81 @@
 
 #include <math.h>
 
+// ------------------------------------------------------------------ router logits
+// z[t][e] = w_router[e] . ln(x[t]) with ln the layer norm of the float32 residual row
+// ((x - mean) / sqrt(var + eps) * weight + bias), all in float32: the router then decides on
+// the unrounded normalised input, whatever dtype the other consumers of the norm take.  One
+// workgroup per token and eight experts; the normalised row waits in LDS.
+template <typename TW>
+__global__ __launch_bounds__(256) void moe_router_logits_kernel(
+    const float* __restrict__ resid, const TW* __restrict__ ln_w, const TW* __restrict__ ln_b,
+    float eps, const TW* __restrict__ w_router, float* __restrict__ z, int W, int E) {
+  extern __shared__ float row_s[];
+  __shared__ float red[4];
+  const int t = blockIdx.x;
+  const float* xr = resid + (long long)t * W;
+  float sum = 0.f;
+  for (int j = threadIdx.x; j < W; j += 256) {
+    const float v = xr[j];
+    row_s[j] = v;
+    sum += v;
+  }
+  const float mean = block_sum<256>(sum, red) / (float)W;
+  float sq = 0.f;
+  for (int j = threadIdx.x; j < W; j += 256) {
+    const float d = row_s[j] - mean;
+    sq += d * d;
+  }
+  const float mult = 1.0f / sqrtf(block_sum<256>(sq, red) / (float)W + eps);
+  for (int j = threadIdx.x; j < W; j += 256)
+    row_s[j] = (row_s[j] - mean) * mult * widen(ln_w[j]) + widen(ln_b[j]);
+  __syncthreads();
+  // a workgroup takes eight experts (grid.y of them cover all), a wave two of them in turn; a
+  // lane's products of a row are asked for eight at a time
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int e_end = min(E, (int)(blockIdx.y + 1) * 8);
+  for (int e = blockIdx.y * 8 + wave; e < e_end; e += 4) {
+    const TW* w = w_router + (long long)e * W;
+    float part[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) part[u] = 0.f;
+    for (int j0 = 0; j0 < W; j0 += 8 * kWave) {
+      TW wv[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int j = j0 + u * kWave + lane;
+        wv[u] = w[j < W ? j : 0];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int j = j0 + u * kWave + lane;
+        part[u] = fmaf(j < W ? row_s[j] : 0.f, widen(wv[u]), part[u]);
+      }
+    }
+    float dot = ((part[0] + part[1]) + (part[2] + part[3])) + ((part[4] + part[5]) + (part[6] + part[7]));
+    dot = wave_sum(dot);
+    if (lane == 0) z[(long long)t * E + e] = dot;
+  }
+}
+
+RLIS_API int rlis_moe_router_logits(const float* resid, const void* ln_w, const void* ln_b,
+                                    float eps, const void* w_router, int dtype, float* z, int T,
+                                    int W, int E, hipStream_t stream) {
+  RLIS_REQUIRE(T >= 0 && W > 0 && W <= 16000 && E > 0 && E <= 8 * 65535,
+               "moe_router_logits: bad sizes");
+  if (T == 0) return 0;
+  if (dtype == RLIS_F32)
+    moe_router_logits_kernel<float><<<dim3(T, ceil_div(E, 8)), 256, (size_t)W * 4, stream>>>(
+        resid, (const float*)ln_w, (const float*)ln_b, eps, (const float*)w_router, z, W, E);
+  else if (dtype == RLIS_BF16)
+    moe_router_logits_kernel<bf16_t><<<dim3(T, ceil_div(E, 8)), 256, (size_t)W * 4, stream>>>(
+        resid, (const bf16_t*)ln_w, (const bf16_t*)ln_b, eps, (const bf16_t*)w_router, z, W, E);
+  else
+    RLIS_REQUIRE(false, "moe_router_logits: unknown dtype %d", dtype);
+  RLIS_LAUNCH_CHECK("moe_router_logits");
+  return 0;
+}
+
 // ------------------------------------------------------------------------ route
 constexpr int kRouteMaxPerLane = 8;      // experts up to 64 * 8
 

@@ -1091,7 +1091,7 @@ from .recurrent import (causal_conv, decay_scan, delta_scan, head_norm_gate,  # 
                         selective_scan, shift_mix, tail_update)
 from .latent import (head_linear, latent_attention, latent_mfma_ok, latent_write,  # noqa: E402,F401
                      sigmoid_gate_)
-from .routed import routed_units, route  # noqa: E402,F401
+from .routed import routed_units, route, router_logits  # noqa: E402,F401
 
 
 def fill_normal(out: torch.Tensor, seed: int, tensor_index: int, mean: float, std: float) -> None:

@@ -35,6 +35,7 @@ _SIGNATURES = {
     "rlis_latent_attention_mfma": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, I, F, I, P, I, I, P],
     "rlis_latent_attention": [P, I, L, P, L, P, P, I, P, P, I, I, I, I, I, F, I, P, P],
     "rlis_sigmoid_gate": [P, L, P, L, I, I, I, P],
+    "rlis_moe_router_logits": [P, P, P, F, P, I, P, I, I, I, P],
     "rlis_moe_route": [P, L, P, I, I, I, I, I, F, P, P, P],
     "rlis_moe_sort": [P, I, I, I, I, P, P, P],
     "rlis_moe_experts": [P, I, L, P, P, P, P, P, I, I, I, I, I, P, P, P],

@@ -22,6 +22,29 @@ SMALL_TILE_MAX_PAIRS = 256
 LARGE_TILE_MIN_PAIRS_PER_EXPERT = 96
 
 
+def router_logits(resid: torch.Tensor, norm_weight: torch.Tensor, norm_bias: torch.Tensor,
+                  eps: float, w_router: torch.Tensor) -> torch.Tensor:
+    """``layer_norm(resid) @ w_router.T`` in float32 from the float32 residual rows ``(T, W)``:
+    the router's logits on the unrounded normalised input.  Norm weight, bias and the router's
+    weight ``(E, W)`` share a dtype (float32 or bfloat16)."""
+    if not resid.is_cuda or resid.dtype != torch.float32 or resid.dim() != 2 \
+            or not resid.is_contiguous():
+        raise KernelError("router_logits: the residual must be contiguous float32 (T, W)")
+    T, W = resid.shape
+    E = w_router.shape[0]
+    for t, shape, what in ((norm_weight, (W,), "norm weight"), (norm_bias, (W,), "norm bias"),
+                           (w_router, (E, W), "router weight")):
+        if tuple(t.shape) != shape or t.dtype != w_router.dtype or not t.is_contiguous() \
+                or t.dtype not in _DT:
+            raise KernelError(f"router_logits: the {what} must be contiguous {shape} of the "
+                              "router weight's dtype")
+    z = torch.empty((T, E), dtype=torch.float32, device=resid.device)
+    lib.call("rlis_moe_router_logits", resid.data_ptr(), norm_weight.data_ptr(),
+             norm_bias.data_ptr(), float(eps), w_router.data_ptr(), _DT[w_router.dtype],
+             z.data_ptr(), T, W, E, lib.stream_ptr())
+    return z
+
+
 def route(logits: torch.Tensor, correction: torch.Tensor, groups: int, keep: int, top: int,
           scale: float) -> Tuple[torch.Tensor, torch.Tensor]:
     """From router logits ``(T, E)`` float32: scores ``s = sigmoid(logits)``, choice scores

@@ -63,7 +63,10 @@ class PreNormBlock(Block):
 class ParallelBlock(Block):
     """Parameters: ``mixer``, ``feed_forward`` (None: the mixer alone), ``norm`` (PartSpecs) and
     ``names``: the weight-name suffix of each under the block's prefix.  The two sublayers'
-    outputs are added in float32 and join the stream as one delta."""
+    outputs are added in float32 and join the stream as one delta.  A feed-forward that sets
+    ``wants_residual`` also gets the float32 residual rows that the norm normalised and the
+    norm itself (``forward(h, step, resid=..., norm=...)``), for decisions that it wants to make
+    on the unrounded input."""
 
     _SLOTS = (("norm", "norm"), ("mixer", "mixer"), ("feed_forward", "feed_forward"))
 
@@ -96,6 +99,10 @@ class ParallelBlock(Block):
         if self.feed_forward is None:
             stream.add(mixed)
             return
-        fed = self.feed_forward.forward(h, step)
+        if getattr(self.feed_forward, "wants_residual", False):
+            # (the norm has folded the pending delta in: stream.x is what it normalised)
+            fed = self.feed_forward.forward(h, step, resid=stream.x, norm=self.norm)
+        else:
+            fed = self.feed_forward.forward(h, step)
         mixed, fed = (d if isinstance(d, torch.Tensor) else d.run() for d in (mixed, fed))
         stream.add(ops.weighted_sum(mixed, 1.0, fed, 1.0, round_parts=stream.round_parts))

@@ -105,9 +105,14 @@ class RoutedSwiGLU(FeedForward):
 
     Tensors under the prefix: ``router`` (experts, W), ``correction`` (experts: added to the
     sigmoid scores for the choice only), ``e<i>.gate|up`` (F, W), ``e<i>.down`` (W, F),
-    ``shared.gate|up|down``.  Router logits, scores and the choice are float32."""
+    ``shared.gate|up|down``.  Router logits, scores and the choice are float32.  A block that
+    hands over the float32 residual rows and the layer norm in front (``wants_residual``) lets
+    the router decide on the unrounded normalised input: the logits then come from one kernel
+    that normalises in float32 itself, and a choice between two close experts does not hang on
+    the rounding of the activations that the experts read."""
 
     graph_safe = True
+    wants_residual = True
 
     @classmethod
     def tensor_specs(cls, params: Dict[str, Any], prefix: str) -> List[TensorSpec]:
@@ -152,8 +157,14 @@ class RoutedSwiGLU(FeedForward):
             self.w_shared_gate_up = torch.cat([gate, up], dim=0).contiguous()
             self.w_shared_down = ctx.take(join(prefix, "shared.down"))
 
-    def forward(self, x: torch.Tensor, step: Any) -> torch.Tensor:
-        logits = ops.linear(x, self.w_router, torch.float32)
+    def forward(self, x: torch.Tensor, step: Any, resid: Any = None, norm: Any = None
+                ) -> torch.Tensor:
+        weight, bias = getattr(norm, "weight", None), getattr(norm, "bias", None)
+        if resid is not None and weight is not None and bias is not None \
+                and weight.dtype == bias.dtype == self.w_router.dtype:
+            logits = ops.router_logits(resid, weight, bias, norm.eps, self.w_router)
+        else:
+            logits = ops.linear(x, self.w_router, torch.float32)
         chosen, weights = ops.route(logits, self.correction, self.groups, self.keep, self.top,
                                     self.scale)
         shared = None

@@ -211,6 +211,13 @@ def sigmoid_gate_(o, g):
 
 
 # ---- routed feed-forward -----------------------------------------------------------------
+def router_logits(resid, norm_weight, norm_bias, eps, w_router):
+    mean = resid.mean(-1, keepdim=True)
+    var = ((resid - mean) ** 2).mean(-1, keepdim=True)
+    h = (resid - mean) / torch.sqrt(var + eps) * norm_weight.float() + norm_bias.float()
+    return h @ w_router.float().t()
+
+
 def route(logits, correction, groups, keep, top, scale):
     T, E = logits.shape
     s = torch.sigmoid(logits)
@@ -403,6 +410,6 @@ def install(monkeypatch) -> None:
                  "causal_conv", "delta_scan", "decay_scan", "head_norm_gate", "selective_scan",
                  "add_layernorm", "scale_", "head_linear", "latent_write", "latent_attention",
                  "latent_mfma_ok",
-                 "sigmoid_gate_", "route", "routed_units"):
+                 "sigmoid_gate_", "route", "routed_units", "router_logits"):
         monkeypatch.setattr(ops, name, globals()[name])
     monkeypatch.setattr(runner, "default_device", lambda: torch.device("cpu"))

@@ -174,6 +174,19 @@ def test_the_choice_of_experts(E, G, keep, top):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T, W, E", [(1, 40, 3), (9, 192, 8), (70, 1000, 33)])
+def test_router_logits_from_the_residual(dtype, T, W, E):
+    """Layer norm and the router's product in one kernel, float32 on weights of either dtype."""
+    from rust_llm_inference_server_amd import ops
+    resid = rnd(T, W, seed=1) * 3 + 0.5
+    w, b = (1 + rnd(W, seed=2, std=0.3)).to(dtype), rnd(W, seed=3, std=0.2).to(dtype)
+    router = rnd(E, W, seed=4, std=W ** -0.5).to(dtype)
+    want = plain.layer_norm(resid.double(), w.double(), b.double(), 1e-5) @ router.double().T
+    got = ops.router_logits(resid.to(DEV), w.to(DEV), b.to(DEV), 1e-5, router.to(DEV))
+    assert got.dtype == torch.float32 and rel(got, want) < 1e-5
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("T, E, top, W, F", [(1, 4, 2, 48, 24), (9, 8, 3, 40, 20),
                                              (200, 6, 2, 64, 32), (77, 3, 1, 36, 12),
                                              (700, 4, 2, 72, 40), (1000, 3, 3, 200, 136)])
