@@ -620,7 +620,8 @@ static LdsGrant g_latent_staged_lds[3];
 
 // Whether the matrix-core kernel takes a latent of R numbers in rows of D.
 RLIS_API int rlis_latent_attention_mfma_ok(int R, int D, int page_size) {
-  return (R > 0 && R <= 4096 && D >= R && D <= 1536 && D % 8 == 0 && page_size % 8 == 0) ? 1 : 0;
+  // (a workgroup's four waves keep 16 query rows of D numbers each in LDS)
+  return (R > 0 && R <= 1024 && D >= R && D <= 1024 && D % 8 == 0 && page_size % 8 == 0) ? 1 : 0;
 }
 
 RLIS_API int rlis_latent_attention_mfma(const void* q, long long ldq, void* out, long long ldo,
