@@ -96,8 +96,6 @@ RLIS_API int rlis_moe_router_logits(const float* resid, const void* ln_w, const 
 }
 
 // ------------------------------------------------------------------------ route
-constexpr int kRouteMaxPerLane = 8;      // experts up to 64 * 8
-
 __device__ __forceinline__ void wave_argmax(float& v, int& idx) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {

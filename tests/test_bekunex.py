@@ -8,7 +8,6 @@ the CPU, where it tests the host logic: run order and shared caches, windows, st
 input tails, the step layout."""
 import copy
 import json
-import os
 
 import pytest
 import torch

@@ -4,8 +4,6 @@ latent's norm / rotation / cache write and the attention over cached latents (wi
 pages in any order), the sigmoid gate, the choice of experts and the routed units (tiles of 16
 and of 64 rows), the selective scan with its state carried over steps, and the convolution's
 bias."""
-import math
-
 import pytest
 import torch
 
