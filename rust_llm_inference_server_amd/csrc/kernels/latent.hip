@@ -683,7 +683,7 @@ RLIS_API int rlis_latent_attention_mfma(const void* q, long long ldq, void* out,
   // sums per wave: up to 128 latent channels in small steps (more workgroups, more loads in
   // flight), up to 256 in large ones (the scores are formed once more per share)
   const int tiles = ceil_div(R, 16);
-  const int nt = tiles <= 4 ? 4 : (tiles <= 8 || split) ? 8 : 16;
+  const int nt = tiles <= 4 ? 4 : (tiles <= 8 || (split && (long long)blocks * heads_y <= 64)) ? 8 : 16;
   dim3 grid(split ? blocks : ceil_div(blocks, 4), heads_y, ceil_div(tiles, nt));
 #define LAUNCH_AS(NT, SP, slot)                                                                \
   do {                                                                                         \

@@ -14,9 +14,11 @@ from .lib import KernelError
 
 _DT = {torch.float32: 0, torch.bfloat16: 1}
 
-# Steps with at most this many (token, expert) pairs take tiles of 16 rows, larger ones of 64: a
-# row's sums are the same either way.
+# Steps with at most this many (token, expert) pairs, or at most 16 pairs per expert on average,
+# take tiles of 16 rows (an expert's weights are then streamed by waves that carry no padding
+# rows through their products), larger ones of 64: a row's sums are the same either way.
 SMALL_TILE_MAX_PAIRS = 256
+SMALL_TILE_MAX_PAIRS_PER_EXPERT = 16
 # bfloat16 steps with at least this many pairs per expert on average take tiles of 128 rows that
 # are staged through LDS (another matrix instruction: a row's sums agree to rounding).
 LARGE_TILE_MIN_PAIRS_PER_EXPERT = 96
@@ -93,7 +95,7 @@ def routed_units(x: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor,
     if T == 0:
         return out
     P = T * top
-    rows = 16 if P <= SMALL_TILE_MAX_PAIRS else 64
+    rows = 16 if P <= max(SMALL_TILE_MAX_PAIRS, SMALL_TILE_MAX_PAIRS_PER_EXPERT * E) else 64
     if x.dtype == torch.bfloat16 and P >= LARGE_TILE_MIN_PAIRS_PER_EXPERT * E and W % 8 == 0 \
             and F % 8 == 0 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0:
         rows = 128
