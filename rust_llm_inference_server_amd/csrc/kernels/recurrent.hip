@@ -1023,34 +1023,60 @@ __device__ __forceinline__ float channel_sum(float v) {
   return v;
 }
 
-template <typename TO, int NPL, int LPC>
+// PASS 0: a workgroup row per sequence, from the slot's state to the slot's state.  The chunked
+// form for long prompts cuts every sequence into chunks of chunk_len tokens (a workgroup row
+// per chunk) and runs three launches: PASS 1 walks every chunk from a zero state and leaves the
+// chunk's end state and the sum of its steps (the product of a chunk's decays is
+// exp(A * that sum)); selective_scan_join walks a sequence's chunks in order,
+// S <- exp(A sum) S + end, from the slot's state, leaves every chunk's true start state where
+// its end state was and the sequence's last state in the slot; PASS 2 walks every chunk again
+// from its start state and makes the outputs.  The recurrence is linear in the state, so this
+// is the sequential walk up to the order of a few additions.
+template <typename TO, int NPL, int LPC, int PASS>
 __global__ __launch_bounds__(256) void selective_scan_kernel(
     TO* __restrict__ out, long long ldo, const TO* __restrict__ x, long long ldx,
     const float* __restrict__ dt_raw, long long lddt, const float* __restrict__ dt_bias,
     const float* __restrict__ bmat, const float* __restrict__ cmat, long long ldbc,
     const float* __restrict__ z, long long ldz, const float* __restrict__ a_log,
     const float* __restrict__ dskip, float* __restrict__ state, long long state_stride,
-    const int* __restrict__ cu, const int* __restrict__ slots, int C, int N) {
-  const int s = blockIdx.y;
+    const int* __restrict__ cu, const int* __restrict__ slots, int C, int N, int num_seqs,
+    int chunk_len, float* __restrict__ chunk_state, float* __restrict__ chunk_dt) {
+  int s = blockIdx.y;
   const int gid = blockIdx.x * blockDim.x + threadIdx.x;
   const int c = gid / LPC, sub = gid % LPC;
   if (c >= C) return;                 // (LPC divides the wave: a channel's lanes stay together)
-  const int t0 = cu[s], t1 = cu[s + 1];
-  float* S = state + (long long)slots[s] * state_stride + (long long)c * N;
+  int t0, t1;
+  if (PASS == 0) {
+    t0 = cu[s];
+    t1 = cu[s + 1];
+  } else {                            // blockIdx.y counts chunks over all sequences
+    int k = blockIdx.y;
+    for (s = 0; s < num_seqs; ++s) {
+      const int chunks = (cu[s + 1] - cu[s] + chunk_len - 1) / chunk_len;
+      if (k < chunks) break;
+      k -= chunks;
+    }
+    if (s == num_seqs) return;
+    t0 = cu[s] + k * chunk_len;
+    t1 = min(t0 + chunk_len, cu[s + 1]);
+  }
+  float* S = PASS == 0 ? state + (long long)slots[s] * state_stride + (long long)c * N
+                       : chunk_state + ((long long)blockIdx.y * C + c) * N;
   float st_[NPL], a[NPL];
 #pragma unroll
   for (int j = 0; j < NPL; ++j) {
     const int n = sub + j * LPC;
-    st_[j] = n < N ? S[n] : 0.f;
+    st_[j] = (PASS != 1 && n < N) ? S[n] : 0.f;
     a[j] = n < N ? -expf(a_log[(long long)c * N + n]) : 0.f;
   }
+  float dt_sum = 0.f;
   const float bias = dt_bias[c], dsk = dskip[c];
   // Tokens are walked in groups of kScanGroup: everything that does not depend on the state
   // (a token's step, input, gate, B and C, and the decays exp(dt A)) is asked for and made for
   // the whole group first, so that the walk itself waits for no load; tokens past the
   // sequence's end take the last token's addresses and are not stored.
   constexpr int G = NPL <= 8 ? 8 : 4;
-  if (t1 - t0 == 1) {                          // a decoded token: nothing to group
+  if (PASS == 0 && t1 - t0 == 1) {             // a decoded token: nothing to group
     const int t = t0;
     const float raw = dt_raw[(long long)t * lddt + c] + bias;
     const float dt = raw > 20.f ? raw : log1pf(expf(raw));
@@ -1095,6 +1121,7 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(
     for (int u = 0; u < G; ++u) {
       if (tg + u < t1) {                       // (the same for all lanes of a sequence)
         const float dt = dtv[u], dx = dt * xv[u];
+        dt_sum += dt;
         float y = 0.f;
 #pragma unroll
         for (int j = 0; j < NPL; ++j) {
@@ -1103,18 +1130,49 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(
           st_[j] = n < N ? v : 0.f;
           y = fmaf(st_[j], cn[u][j], y);
         }
-        y = channel_sum<LPC>(y);
-        if (sub == 0)
-          st(out + (long long)(tg + u) * ldo + c,
-             (y + dsk * xv[u]) * (zv[u] / (1.0f + expf(-zv[u]))));
+        if (PASS != 1) {
+          y = channel_sum<LPC>(y);
+          if (sub == 0)
+            st(out + (long long)(tg + u) * ldo + c,
+               (y + dsk * xv[u]) * (zv[u] / (1.0f + expf(-zv[u]))));
+        }
       }
     }
   }
+  if (PASS == 2) return;               // (the join has left the sequence's last state in the slot)
 #pragma unroll
   for (int j = 0; j < NPL; ++j) {
     const int n = sub + j * LPC;
     if (n < N) S[n] = st_[j];
   }
+  if (PASS == 1 && sub == 0) chunk_dt[(long long)blockIdx.y * C + c] = dt_sum;
+}
+
+// One thread per (sequence, channel, state): the sequence's chunks in order.
+__global__ void selective_scan_join_kernel(float* __restrict__ state, long long state_stride,
+                                           const float* __restrict__ a_log,
+                                           float* __restrict__ chunk_state,
+                                           const float* __restrict__ chunk_dt,
+                                           const int* __restrict__ cu,
+                                           const int* __restrict__ slots, int C, int N,
+                                           int chunk_len) {
+  const int s = blockIdx.y;
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (long long)C * N) return;
+  const int c = (int)(i / N);
+  int first = 0;
+  for (int q = 0; q < s; ++q) first += (cu[q + 1] - cu[q] + chunk_len - 1) / chunk_len;
+  const int chunks = (cu[s + 1] - cu[s] + chunk_len - 1) / chunk_len;
+  float* slot = state + (long long)slots[s] * state_stride + i;
+  const float a = -expf(a_log[i]);
+  float S = *slot;
+  for (int k = 0; k < chunks; ++k) {
+    float* at = chunk_state + (long long)(first + k) * C * N + i;
+    const float end = *at;
+    *at = S;
+    S = expf(a * chunk_dt[(long long)(first + k) * C + c]) * S + end;
+  }
+  *slot = S;
 }
 
 RLIS_API int rlis_selective_scan(void* out, int out_dtype, long long ldo, const void* x,
@@ -1123,7 +1181,9 @@ RLIS_API int rlis_selective_scan(void* out, int out_dtype, long long ldo, const 
                                  long long ldbc, const float* z, long long ldz,
                                  const float* a_log, const float* dskip, float* state,
                                  long long state_stride, const int* cu, const int* slots,
-                                 int num_seqs, int C, int N, int long_runs, hipStream_t stream) {
+                                 int num_seqs, int C, int N, int long_runs, int chunk_len,
+                                 int max_chunks, float* chunk_state, float* chunk_dt,
+                                 hipStream_t stream) {
   RLIS_REQUIRE(num_seqs >= 0 && C > 0 && N > 0, "selective_scan: bad sizes C=%d N=%d", C, N);
   RLIS_REQUIRE(N <= 1024, "selective_scan: a state of %d numbers per channel is too large", N);
   RLIS_REQUIRE(ldo >= C && ldx >= C && lddt >= C && ldz >= C && ldbc >= N &&
@@ -1131,10 +1191,26 @@ RLIS_API int rlis_selective_scan(void* out, int out_dtype, long long ldo, const 
                "selective_scan: strides shorter than rows");
   RLIS_REQUIRE(num_seqs <= 65535, "selective_scan: too many sequences");
   if (num_seqs == 0) return 0;
+  RLIS_REQUIRE(chunk_len == 0 || (chunk_len > 0 && max_chunks > 0 && max_chunks <= 65535 &&
+                                  chunk_state && chunk_dt),
+               "selective_scan: the chunked form needs its scratch and at most 65,535 chunks");
+#define LAUNCH_PASS(TO, NPL, LPC, PASS, ROWS)                                                 \
+  selective_scan_kernel<TO, NPL, LPC, PASS>                                                   \
+      <<<dim3(ceil_div(C * LPC, 256), ROWS), 256, 0, stream>>>(                               \
+          (TO*)out, ldo, (const TO*)x, ldx, dt_raw, lddt, dt_bias, bmat, cmat, ldbc, z, ldz,  \
+          a_log, dskip, state, state_stride, cu, slots, C, N, num_seqs, chunk_len,            \
+          chunk_state, chunk_dt)
 #define LAUNCH(TO, NPL, LPC)                                                                  \
-  selective_scan_kernel<TO, NPL, LPC><<<dim3(ceil_div(C * LPC, 256), num_seqs), 256, 0, stream>>>( \
-      (TO*)out, ldo, (const TO*)x, ldx, dt_raw, lddt, dt_bias, bmat, cmat, ldbc, z, ldz, a_log, dskip,   \
-      state, state_stride, cu, slots, C, N)
+  do {                                                                                        \
+    if (chunk_len > 0) {                                                                      \
+      LAUNCH_PASS(TO, NPL, LPC, 1, max_chunks);                                               \
+      selective_scan_join_kernel<<<dim3(ceil_div(C * N, 256), num_seqs), 256, 0, stream>>>(   \
+          state, state_stride, a_log, chunk_state, chunk_dt, cu, slots, C, N, chunk_len);     \
+      LAUNCH_PASS(TO, NPL, LPC, 2, max_chunks);                                               \
+    } else {                                                                                  \
+      LAUNCH_PASS(TO, NPL, LPC, 0, num_seqs);                                                 \
+    }                                                                                         \
+  } while (0)
   // long_runs: sequences bring many tokens each and there are few of them, so a channel's states
   // are spread over more lanes (more waves on a chip that the walk leaves mostly idle); the sum
   // over the states is then added up in another order
@@ -1153,6 +1229,7 @@ RLIS_API int rlis_selective_scan(void* out, int out_dtype, long long ldo, const 
   else RLIS_REQUIRE(false, "selective_scan: unknown dtype %d", out_dtype);
 #undef BY_N
 #undef LAUNCH
+#undef LAUNCH_PASS
   RLIS_LAUNCH_CHECK("selective_scan");
   return 0;
 }

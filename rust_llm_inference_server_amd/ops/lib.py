@@ -27,7 +27,8 @@ _SIGNATURES = {
     "rlis_shift_mix": [P, P, I, P, P, L, P, P, P, I, I, I, P],
     "rlis_tail_update": [P, L, P, I, L, I, I, P, P, I, P],
     "rlis_causal_conv": [P, I, P, L, P, P, I, I, P, L, P, P, P, I, I, I, I, F, F, I, P],
-    "rlis_selective_scan": [P, I, L, P, L, P, L, P, P, P, L, P, L, P, P, P, L, P, P, I, I, I, I, P],
+    "rlis_selective_scan": [P, I, L, P, L, P, L, P, P, P, L, P, L, P, P, P, L, P, P, I, I, I, I, I, I,
+                            P, P, P],
     "rlis_add_layernorm": [P, P, I, P, P, I, P, I, P, I, I, F, I, I, L, I, F, P],
     "rlis_scale": [P, I, L, F, P],
     "rlis_head_linear": [P, I, L, I, P, P, I, L, I, I, I, I, I, P],

@@ -225,6 +225,14 @@ def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, he
 # host: the number of rows and of sequences).
 SPREAD_SCAN_MIN_MEAN_TOKENS = 64
 SPREAD_SCAN_MAX_CHANNELS = 65536
+# A step of at least CHUNKED_SCAN_MIN_TOKENS tokens whose sequences bring at least
+# CHUNKED_SCAN_MIN_MEAN_TOKENS each on average walks chunks of CHUNKED_SCAN_LEN tokens side by
+# side: every chunk from a zero state, the chunks' states joined in order, every chunk again from
+# its true start state (the recurrence is linear in the state).  The result agrees with the
+# sequential walk to rounding.
+CHUNKED_SCAN_MIN_TOKENS = 512
+CHUNKED_SCAN_MIN_MEAN_TOKENS = 128
+CHUNKED_SCAN_LEN = 64
 
 
 def selective_scan(x: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, b: torch.Tensor,
@@ -253,12 +261,21 @@ def selective_scan(x: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor,
         raise KernelError("selective_scan: operand shapes do not match the channels and states")
     stride = _state(state, C * N, "selective_scan")
     out = torch.empty((T, C), dtype=x.dtype, device=x.device)
+    chunk_len = max_chunks = 0
+    chunk_state = chunk_dt = None
+    if T >= CHUNKED_SCAN_MIN_TOKENS and T >= CHUNKED_SCAN_MIN_MEAN_TOKENS * max(1, num_seqs):
+        chunk_len = int(CHUNKED_SCAN_LEN)
+        max_chunks = -(-T // chunk_len) + num_seqs          # an upper bound, known on the host
+        chunk_state = torch.empty((max_chunks, C * N), dtype=torch.float32, device=x.device)
+        chunk_dt = torch.empty((max_chunks, C), dtype=torch.float32, device=x.device)
     lib.call("rlis_selective_scan", out.data_ptr(), _dt(out), C, x.data_ptr(), ldx,
              dt_raw.data_ptr(), lddt, _vec(dt_bias, C, "selective_scan dt bias"), b.data_ptr(),
              c.data_ptr(), ldbc, z.data_ptr(), ldz, _vec(a_log.reshape(-1), C * N,
                                                          "selective_scan A_log"),
              _vec(skip, C, "selective_scan skip"), state.data_ptr(), stride,
              _meta(cu, num_seqs + 1, "cu"), _meta(slots, num_seqs, "slots"), num_seqs, C, N,
-             int(T >= SPREAD_SCAN_MIN_MEAN_TOKENS * max(1, num_seqs)
-                 and num_seqs * C <= SPREAD_SCAN_MAX_CHANNELS), lib.stream_ptr())
+             int(chunk_len == 0 and T >= SPREAD_SCAN_MIN_MEAN_TOKENS * max(1, num_seqs)
+                 and num_seqs * C <= SPREAD_SCAN_MAX_CHANNELS), chunk_len, max_chunks,
+             None if chunk_state is None else chunk_state.data_ptr(),
+             None if chunk_dt is None else chunk_dt.data_ptr(), lib.stream_ptr())
     return out

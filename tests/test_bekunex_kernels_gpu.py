@@ -217,10 +217,18 @@ def test_routed_units(dtype, T, E, top, W, F):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("C, N", [(24, 5), (64, 16), (40, 20), (33, 64), (16, 70), (8, 300)])
-def test_selective_scan_carries_its_state(dtype, C, N):
+@pytest.mark.parametrize("chunked", [False, True])
+def test_selective_scan_carries_its_state(dtype, C, N, chunked, monkeypatch):
     """Two sequences in one step, then their continuations in a second step with the slots
-    swapped in the batch's order: the same as each sequence in one pass."""
+    swapped in the batch's order: the same as each sequence in one pass.  ``chunked``: the form
+    for long prompts, here with chunks of 4 tokens, so that sequences of 2 to 13 tokens are
+    one chunk, several whole ones, and some with a short last one."""
     from rust_llm_inference_server_amd import ops
+    from rust_llm_inference_server_amd.ops import recurrent
+    if chunked:
+        monkeypatch.setattr(recurrent, "CHUNKED_SCAN_MIN_TOKENS", 0)
+        monkeypatch.setattr(recurrent, "CHUNKED_SCAN_MIN_MEAN_TOKENS", 0)
+        monkeypatch.setattr(recurrent, "CHUNKED_SCAN_LEN", 4)
     lens = [(9, 6), (2, 13)]
     total = [a + b for a, b in lens]
     data = []
