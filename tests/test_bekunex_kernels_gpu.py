@@ -285,3 +285,37 @@ def test_the_convolutions_bias_and_output_dtype():
         got = ops.causal_conv(x.to(DEV), taps.to(DEV), state, meta([0] * T), meta([0, T]),
                               meta([0]), 1, bias=bias.to(DEV), out_dtype=dtype)
         assert got.dtype == dtype and rel(got, plain.silu(acc)) < TOL[dtype]
+
+
+@pytest.mark.parametrize("H, d, r, R, window", [(16, 16, 16, 128, None), (32, 8, 0, 288, 300),
+                                                (3, 32, 0, 64, 77)])
+def test_large_steps_of_both_attention_kernels_agree(H, d, r, R, window, monkeypatch):
+    """Two sequences of 1,100 and 500 tokens in one step, behind 40 cached positions of the first:
+    the matrix-core kernel in the forms it chooses by itself for a step of this size (staged, or
+    a wave per block) against the vector-unit kernel, row by row."""
+    from rust_llm_inference_server_amd import ops
+    from rust_llm_inference_server_amd.ops import latent
+    dtype, page, D = torch.bfloat16, 16, R + r
+    lens, starts = [1100, 500], [40, 0]
+    total = [a + b for a, b in zip(lens, starts)]
+    T = sum(lens)
+    pages_needed = [-(-n // page) for n in total]
+    num_pages = sum(pages_needed) + 3
+    perm = torch.randperm(num_pages, generator=torch.Generator().manual_seed(5))
+    table = torch.zeros(2, 128, dtype=torch.int32)
+    table[0, :pages_needed[0]] = perm[:pages_needed[0]].to(torch.int32)
+    table[1, :pages_needed[1]] = perm[pages_needed[0]:sum(pages_needed)].to(torch.int32)
+    pages = (rnd(num_pages, page, D, seed=11) * 0.7).to(dtype).to(DEV)
+    pages_t = pages[:, :, :R].transpose(1, 2).contiguous()
+    q = (rnd(T, H * D, seed=12) * 0.5).to(dtype).to(DEV)
+    seq = torch.cat([torch.zeros(lens[0]), torch.ones(lens[1])]).to(torch.int32).to(DEV)
+    pos = torch.cat([torch.arange(starts[0], total[0]),
+                     torch.arange(starts[1], total[1])]).to(torch.int32).to(DEV)
+    cu = torch.tensor([0, lens[0], T], dtype=torch.int32, device=DEV)
+    sink = (rnd(H, seed=13)).to(DEV)
+    args = (q, pages, table.to(DEV), seq, pos, H, R, 0.2, window, sink)
+    want = ops.latent_attention(*args)
+    for staged in (True, False):
+        monkeypatch.setattr(latent, "LATENT_STAGED", staged)
+        got = ops.latent_attention(*args, pages_t=pages_t, cu=cu, num_seqs=2)
+        assert rel(got, want) < 2e-2
